@@ -12,8 +12,8 @@ Beside it, in the same run:
     attention over the KV cache, fc1 + GELU, out_proj, fc2, residual adds; 100,769,792 bytes of weights and vectors
     plus the layer's K/V prefix per launch, 24 launches per token), timed per launch with HIP event pairs on the
     library's stream inside the same greedy loop, right after the timed steps;
-  * extra: config 1's stand-alone GEMV [1x2048].[2048x8192] (33,591,296 bytes per launch, rotating over 24 weight
-    buffers so the 256 MB last-level cache cannot serve them), the vision fc1/fc2 GEMMs (729x1152x4304, 729x4304x1152), decode / prefill / vision attention and the
+  * extra: config 1's stand-alone GEMV [1x2048].[2048x8192] (33,591,296 bytes per launch, rotating over 32 weight
+    buffers = 1 GiB so the 256 MB last-level cache cannot serve them, with a plain read of the same bytes beside it), the vision fc1/fc2 GEMMs (729x1152x4304, 729x4304x1152), decode / prefill / vision attention and the
     full 27-block vision encoder, each with its own roofline fraction;
   * cpu_baseline: a CPU restatement of the reference's kernels (same blocking and threading as the Zig code; the
     Zig toolchain is not available) timed on this host on a bounded sample of the same decode workload.
@@ -176,10 +176,12 @@ def profile_decode_kernels(model, us_per_token, mode=None):
     return out
 
 
-def bench_gemv(moon, ctx, iters=240):
-    """Config 1 shape with the decode step's fused epilogue, rotating over distinct weight buffers."""
+def bench_gemv(moon, ctx, iters=256):
+    """Config 1: y = f16(f16(x.W^T) + b), x [1,2048], W [8192,2048], rotating over 32 distinct weight buffers (1 GiB) so that
+    the 256 MB last-level cache cannot serve them.  Beside it the plain-read kernel on the same buffers: what one launch
+    that only streams 33.6 MB reaches on this device."""
     L_ = moon._lib
-    N, K, ring = FFN, D, 24
+    N, K, ring = FFN, D, 32
     w = ctx.alloc(ring * N * K * 2)
     for i in range(ring):
         w.fill_normal(N * K, 0, 100 + i, 0.02, byte_offset=i * N * K * 2)
@@ -191,14 +193,19 @@ def bench_gemv(moon, ctx, iters=240):
 
     def launch(i):
         ctx.check(ctx.lib.moon_dev_linear(ctx.handle, x.ptr, 1, K, w.offset((i % ring) * N * K * 2), N, L_.B_NK, b.ptr,
-                                          L_.EPI_BIAS_GELU, y.ptr))
+                                          L_.EPI_BIAS, y.ptr))
+
+    def read(i):
+        ctx.check(ctx.lib.moon_dev_read(ctx.handle, w.offset((i % ring) * N * K * 2), N * K * 2, None))
 
     us = event_time_us(ctx, launch, iters)
+    us_read = event_time_us(ctx, read, iters)
     alg_bytes = N * K * 2 + K * 2 + N * 2 + N * 2
     for buf in (w, x, b, y):
         buf.free()
-    return dict(kernel="gemv_nt_kernel<2,4,BIAS_GELU> [1x2048].[2048x8192]^T", us=us, bytes=alg_bytes, gbs=alg_bytes / us / 1e3,
-                frac=alg_bytes / us / 1e3 / HBM_PEAK_GBS, ring_mib=ring * N * K * 2 / 2**20)
+    return dict(kernel="gemv_nt_kernel<2,4,BIAS> [1x2048].[2048x8192]^T + bias", us=us, bytes=alg_bytes, gbs=alg_bytes / us / 1e3,
+                frac=alg_bytes / us / 1e3 / HBM_PEAK_GBS, ring_mib=ring * N * K * 2 / 2**20,
+                plain_read_same_bytes=dict(us=us_read, gbs=N * K * 2 / us_read / 1e3, frac=N * K * 2 / us_read / 1e3 / HBM_PEAK_GBS))
 
 
 def bench_gemm(moon, ctx, M, K, N, iters=50):

@@ -177,6 +177,10 @@ int moon_dev_download(moon_ctx *ctx, void *host, const void *dptr, size_t bytes)
 /* Device-to-device copy by a plain kernel (bytes and both pointers multiples of 16); asynchronous on the context's
  * stream.  Its traffic is exactly `bytes` read + `bytes` written, which makes it the yardstick for counter readings. */
 int moon_dev_copy(moon_ctx *ctx, void *dst, const void *src, size_t bytes);
+/* Plain read of `bytes` (a multiple of 16, like the pointer) by a kernel that does nothing else; sink may be NULL or
+ * point to 4 device bytes (never written for ordinary data).  No counterpart in the reference: it is the yardstick for
+ * what one launch that streams this many bytes from HBM can reach on the device at hand. */
+int moon_dev_read(moon_ctx *ctx, const void *src, size_t bytes, void *sink);
 /* Deterministic synthetic data, bit-identical to the test generator on the host:
  * f16 ~N(0,std) (Irwin-Hall over splitmix64 counters) and uniform u32 in [0,modulo). */
 int moon_dev_fill_normal_f16(moon_ctx *ctx, void *dptr, size_t n, uint64_t seed, uint64_t stream, float std_dev);
@@ -198,6 +202,10 @@ int moon_dev_sdpa(moon_ctx *ctx, const void *q, const void *k, const void *v, vo
  * (q | k | v, text_model.zig:198-226); out is [n_heads*head_dim] (already head-merged, :293-294). */
 int moon_dev_decode_attention(moon_ctx *ctx, const void *qkv, void *cache_k, void *cache_v, const void *freqs_cis,
                               void *out, size_t n_heads, size_t head_dim, size_t rot_dim, size_t max_seq, size_t pos);
+/* rope.precomputeFreqsCis(f32, dim, end, theta) (rope.zig:32-128) on the device: table[end, rot_dim/2, 2] f32 of
+ * (cos, sin)(p * theta^(-2i/rot_dim)), the table the text session builds for itself (text_model.zig:88) and
+ * moon_dev_decode_attention reads.  rot_dim odd or zero -> MOON_EROT_DIM. */
+int moon_dev_rope_table(moon_ctx *ctx, void *table, size_t rot_dim, size_t end, float theta);
 int moon_dev_layernorm(moon_ctx *ctx, const void *x, const void *gamma, const void *beta, void *y,
                        size_t rows, size_t dim, float eps);
 /* moon_sample on logits that already sit in HBM; the index comes back to the host. */
@@ -267,6 +275,12 @@ int moon_text_greedy_profile(moon_text_model *m, size_t n_steps, uint32_t *out_i
  * 3 = two kernels per layer (LayerNorm + qkv + fc1 + attention; out_proj + fc2 + residual).  All produce the same bits.
  * A wait that expires makes the call return MOON_EHIP. */
 int moon_text_set_decode_mode(moon_text_model *m, int mode);
+/* After a MOON_EHIP from moon_text_greedy / moon_text_sample caused by an expired wait inside a fused decode kernel the
+ * session refuses further forward / greedy / sample calls until moon_text_reset: workgroups that gave up may have skipped
+ * the cache append of their position.  moon_text_reset then also restarts the kernels' counters.
+ * moon_text_debug_raise_wait_error sets the error word those waits look at, as an expired wait does (a test hook for
+ * that path; no counterpart in the reference, whose ops cannot fail this way). */
+int moon_text_debug_raise_wait_error(moon_text_model *m);
 /* current KV length */
 size_t moon_text_position(const moon_text_model *m);
 /* Copy of the last forward's hidden states [n, dim] (n = tokens of that forward). */

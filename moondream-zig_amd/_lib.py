@@ -95,12 +95,14 @@ SIGNATURES = {
     "moon_dev_upload": (_i, [_vp, _vp, _vp, _sz]),
     "moon_dev_download": (_i, [_vp, _vp, _vp, _sz]),
     "moon_dev_copy": (_i, [_vp, _vp, _vp, _sz]),
+    "moon_dev_read": (_i, [_vp, _vp, _sz, _vp]),
     "moon_dev_fill_normal_f16": (_i, [_vp, _vp, _sz, _u64, _u64, _f]),
     "moon_dev_fill_const_f16": (_i, [_vp, _vp, _sz, _f]),
     "moon_dev_fill_uniform_u32": (_i, [_vp, _vp, _sz, _u64, _u64, _u32]),
     "moon_dev_linear": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _i, _vp, _i, _vp]),
     "moon_dev_sdpa": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _l, _vp, _sz]),
     "moon_dev_decode_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]),
+    "moon_dev_rope_table": (_i, [_vp, _vp, _sz, _sz, _f]),
     "moon_dev_layernorm": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _f]),
     "moon_timer_start": (_i, [_vp]),
     "moon_timer_stop": (_i, [_vp, C.POINTER(_f)]),
@@ -115,6 +117,7 @@ SIGNATURES = {
     "moon_text_sample": (_i, [_vp, _vp, _vp, _sz, _vp]),
     "moon_text_greedy_profile": (_i, [_vp, _sz, _vp, _vp, _vp]),
     "moon_text_set_decode_mode": (_i, [_vp, _i]),
+    "moon_text_debug_raise_wait_error": (_i, [_vp]),
     "moon_text_position": (_sz, [_vp]),
     "moon_text_hidden": (_i, [_vp, _vp, _sz]),
     "moon_text_weight_bytes_per_token": (_sz, [_vp]),

@@ -356,6 +356,15 @@ extern "C" int moon_dev_decode_attention(moon_ctx *ctx, const void *qkv, void *c
                                    (half_t *)out, n_heads, head_dim, rot_dim, max_seq, pos, nullptr);
 }
 
+extern "C" int moon_dev_rope_table(moon_ctx *ctx, void *table, size_t rot_dim, size_t end, float theta) {
+    if (!ctx) return MOON_EINVAL;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (!table) return moon_fail(ctx, MOON_EINVAL, "dev_rope_table: null table");
+    if (!rot_dim || rot_dim % 2) return moon_fail(ctx, MOON_EROT_DIM, "dev_rope_table: rot_dim %zu must be even and positive", rot_dim);
+    if (rot_dim / 2 * end > 0x7fffffffull) return moon_fail(ctx, MOON_EINVAL_DIM, "dev_rope_table: table too large");
+    return launch_rope_table(ctx, (float *)table, rot_dim, end, theta);
+}
+
 extern "C" int moon_dev_layernorm(moon_ctx *ctx, const void *x, const void *gamma, const void *beta, void *y, size_t rows,
                                   size_t dim, float eps) {
     if (!ctx) return MOON_EINVAL;

@@ -274,6 +274,42 @@ extern "C" int moon_dev_copy(moon_ctx *ctx, void *dst, const void *src, size_t b
     return MOON_OK;
 }
 
+// Plain read of n16 * 16 bytes, eight 16-byte non-temporal loads in flight per lane, 1024 workgroups: what this device
+// gives a kernel that does nothing but stream `bytes` from HBM in one launch -- the ceiling beside which a
+// bandwidth-bound kernel of the same size is read.  The xor of everything lands in sink[0] only if it is a value that
+// random data does not produce, so the loads stay and nothing is written.
+typedef unsigned int read_u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void read16_kernel(const read_u32x4 *__restrict__ src, size_t n16, uint32_t *sink) {
+    const size_t stride = size_t(gridDim.x) * blockDim.x;
+    size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    uint32_t acc = 0;
+    for (; i + 7 * stride < n16; i += 8 * stride) {
+        read_u32x4 v[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) v[k] = __builtin_nontemporal_load(src + i + k * stride);
+#pragma unroll
+        for (int k = 0; k < 8; k++) acc ^= v[k][0] ^ v[k][1] ^ v[k][2] ^ v[k][3];
+    }
+    for (; i < n16; i += stride) {
+        const read_u32x4 v = __builtin_nontemporal_load(src + i);
+        acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
+    }
+    if (acc == 0x9e3779b9u && sink) sink[0] = acc;
+}
+
+extern "C" int moon_dev_read(moon_ctx *ctx, const void *src, size_t bytes, void *sink) {
+    if (!ctx || (!src && bytes)) return moon_fail(ctx, MOON_EINVAL, "read: null pointer");
+    if (bytes % 16 || (uintptr_t)src % 16) return moon_fail(ctx, MOON_EINVAL, "read: pointer and size must be multiples of 16");
+    if (!bytes) return MOON_OK;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    MOON_HIP(ctx, hipSetDevice(ctx->device));
+    const size_t n16 = bytes / 16, want = (n16 + 255) / 256;
+    const unsigned grid = (unsigned)(want < 1024 ? want : 1024);
+    hipLaunchKernelGGL(read16_kernel, dim3(grid), dim3(256), 0, ctx->stream, (const read_u32x4 *)src, n16, (uint32_t *)sink);
+    MOON_HIP(ctx, hipGetLastError());
+    return MOON_OK;
+}
+
 extern "C" int moon_dev_fill_normal_f16(moon_ctx *ctx, void *dptr, size_t n, uint64_t seed, uint64_t stream, float std_dev) {
     if (!ctx || (!dptr && n)) return moon_fail(ctx, MOON_EINVAL, "fill: null pointer");
     std::lock_guard<std::mutex> lock(ctx->mu);

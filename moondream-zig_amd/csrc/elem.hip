@@ -94,16 +94,19 @@ __global__ void embed_kernel(const half_t *__restrict__ wte, const uint32_t *__r
     for (int i = threadIdx.x; i < dim; i += blockDim.x) dst[i] = src[i];
 }
 
-// rope.precomputeFreqsCis (rope.zig:32-128): [end, rot_dim/2, 2] f32 (cos, sin)
+// rope.precomputeFreqsCis (rope.zig:32-128): [end, rot_dim/2, 2] f32 (cos, sin).  The reference's steps are f32: power =
+// 2i/dim, inv = 1/pow(theta, power), angle = p * inv, then cos and sin.  An f32 pow that is one ulp off moves the angle of
+// the last rows by 1e-4 rad, so each transcendental is evaluated in f64 on its f32 argument and rounded once: the
+// correctly rounded f32 result (32768 entries, once per model).
 __global__ void rope_table_kernel(float *table, int half_pairs, int end, int dim, float theta) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= half_pairs * end) return;
     const int p = i / half_pairs, f = i % half_pairs;
     const float power = (float)(2 * f) / (float)dim;
-    const float inv = 1.0f / powf(theta, power);
+    const float inv = 1.0f / (float)pow((double)theta, (double)power);
     const float ang = (float)p * inv;
-    table[2 * i] = cosf(ang);
-    table[2 * i + 1] = sinf(ang);
+    table[2 * i] = (float)cos((double)ang);
+    table[2 * i + 1] = (float)sin((double)ang);
 }
 
 __device__ __forceinline__ void rotate_pair(float xr, float xi, float c, float s, half_t &o_r, half_t &o_i) {

@@ -91,6 +91,7 @@ struct moon_text_model {
     float *u_dev = nullptr;        // [max_seq] the sampling loop's random numbers, one per step
     uint32_t *state_dev = nullptr; // [0] = position (KV length), [1] = step counter, [2] = current token
     size_t cur_len = 0, last_n = 0;
+    bool cache_invalid = false;    // a fused decode kernel gave up on a wait: positions may be missing from the cache until moon_text_reset
     // persistent decode kernel state
     int decode_mode = 0;           // 0: a few fused kernels per layer (default); 1: one persistent kernel for the whole greedy loop
     int groups = 0;                // co-resident workgroups of the persistent kernel (0: unavailable)
@@ -227,6 +228,23 @@ void free_all(moon_text_model *m) {
     (void)hipStreamSynchronize(m->ctx->stream);
     for (void *p : m->allocs) (void)hipFree(p);
     m->allocs.clear();
+}
+
+// Counters, exchange buffers and error words of the fused decode kernels back to their initial state (fill kernels in
+// stream order, no memset), and the host's launch counts with them.  A kernel that gave up on a wait leaves counters
+// short of the targets the host has already moved on to; nothing that is cleared here survives such a launch.
+int clear_sync_state(moon_text_model *m) {
+    const Sizes z = sizes(m->cfg);
+    moon_ctx *ctx = m->ctx;
+    MOON_TRY(launch_fill_uniform_u32(ctx, m->head_count, z.L * z.H, 0, 0, 1));
+    MOON_TRY(launch_fill_uniform_u32(ctx, m->front_sync, z.L * z.H * 32 + 1, 0, 0, 1));
+    MOON_TRY(launch_fill_uniform_u32(ctx, m->layer_sync, z.L * m->layer_sync_words + 1, 0, 0, 1));
+    MOON_TRY(launch_fill_uniform_u32(ctx, m->lm_exchange, decode_lm_head_words(ctx), 0, 0, 1));
+    m->attn_launches.assign(z.L, 0);
+    m->front_launches.assign(z.L, 0);
+    m->layer_launches.assign(z.L, 0);
+    m->lm_launches = 0;
+    return MOON_OK;
 }
 
 struct ProfScope {
@@ -459,6 +477,9 @@ extern "C" int moon_text_reset(moon_text_model *m) {
     std::lock_guard<std::mutex> lock(m->ctx->mu);
     m->cur_len = 0;
     m->last_n = 0;
+    MOON_HIP(m->ctx, hipSetDevice(m->ctx->device));
+    if (m->cache_invalid) MOON_TRY(clear_sync_state(m)); // after a failed wait: counters and targets start over together
+    m->cache_invalid = false;
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, m->ctx->stream, m->state_dev, 0u, 0u);
     MOON_HIP(m->ctx, hipGetLastError());
     return MOON_OK;
@@ -472,6 +493,7 @@ extern "C" int moon_text_forward(moon_text_model *m, const uint32_t *ids, size_t
     std::lock_guard<std::mutex> lock(ctx->mu);
     if (!ids && n_ids) return moon_fail(ctx, MOON_EINVAL, "text_forward: null ids");
     if (!n_ids) return moon_fail(ctx, MOON_EINVAL_DIM, "text_forward: empty input (InvalidInputShape)");
+    if (m->cache_invalid) return moon_fail(ctx, MOON_EHIP, "text_forward: an earlier decode call failed; call moon_text_reset first");
     if (m->cur_len + n_ids > m->cfg.max_seq)
         return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "text_forward: %zu + %zu tokens > max_seq %zu (SequenceTooLong)", m->cur_len, n_ids, m->cfg.max_seq);
     for (size_t i = 0; i < n_ids; i++)
@@ -548,6 +570,7 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
                          const float *u = nullptr) {
     moon_ctx *ctx = m->ctx;
     if (!out_ids && n_steps) return moon_fail(ctx, MOON_EINVAL, "text_greedy: null output");
+    if (m->cache_invalid) return moon_fail(ctx, MOON_EHIP, "text_greedy: an earlier decode call failed; call moon_text_reset first");
     if (!m->last_n) return moon_fail(ctx, MOON_EINVAL, "text_greedy: no prefill yet");
     if (!n_steps) return MOON_OK;
     if (m->cur_len + n_steps > m->cfg.max_seq)
@@ -664,8 +687,6 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
             p.kinds.clear();
         }
     }
-    m->cur_len += n_steps;
-    m->last_n = 1;
     uint32_t front_error = 0;
     MOON_HIP(ctx, hipMemcpyAsync(out_ids, m->ids_dev, n_steps * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
     if (use_layer)
@@ -674,7 +695,16 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
     if (use_front)
         MOON_HIP(ctx, hipMemcpyAsync(&front_error, m->front_sync + m->cfg.n_layers * m->cfg.n_heads * 32, sizeof(front_error), hipMemcpyDeviceToHost, ctx->stream));
     MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    if (front_error != 0) return moon_fail(ctx, MOON_EHIP, "fused decode kernel: a wait between its phases timed out");
+    if (front_error != 0) {
+        // Workgroups that gave up skipped their counter updates and the cache append of their position: the counters
+        // are cleared here, the cache and the position stay unusable until moon_text_reset.
+        m->cache_invalid = true;
+        m->last_n = 0;
+        (void)clear_sync_state(m);
+        return moon_fail(ctx, MOON_EHIP, "fused decode kernel: a wait between its phases timed out; the session needs moon_text_reset");
+    }
+    m->cur_len += n_steps;
+    m->last_n = 1;
     if (use_layer && m->layer_trace) print_layer_trace(m);
     return MOON_OK;
 }
@@ -719,6 +749,22 @@ extern "C" int moon_text_greedy_profile(moon_text_model *m, size_t n_steps, uint
         launches[k] = prof.count[k];
         avg_us[k] = prof.count[k] ? (float)(prof.sum_ms[k] * 1e3 / (double)prof.count[k]) : 0.f;
     }
+    return MOON_OK;
+}
+
+// Raises the error word that the fused decode kernels' waits look at, as a kernel does when its wait expires.  For tests
+// of the recovery path: every kernel still runs to its end, a workgroup that has to poll a counter for long leaves early.
+extern "C" int moon_text_debug_raise_wait_error(moon_text_model *m) {
+    if (!m) return MOON_EINVAL;
+    moon_ctx *ctx = m->ctx;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    const Sizes z = sizes(m->cfg);
+    MOON_HIP(ctx, hipSetDevice(ctx->device));
+    // the word before each error word is the unused tail of a counter line: writes {0, 1} to (tail, error word)
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->layer_sync + z.L * m->layer_sync_words - 1, 0u, 1u);
+    MOON_HIP(ctx, hipGetLastError());
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->front_sync + z.L * z.H * 32 - 1, 0u, 1u);
+    MOON_HIP(ctx, hipGetLastError());
     return MOON_OK;
 }
 

@@ -18,6 +18,19 @@ def precompute_freqs_cis(dim: int, end: int, theta: float = 10000.0) -> np.ndarr
     return np.stack([np.cos(ang, dtype=np.float32), np.sin(ang, dtype=np.float32)], axis=-1).astype(np.float32)
 
 
+def precompute_freqs_cis_device(dim: int, end: int, theta: float = 10000.0, ctx: Context | None = None) -> np.ndarray:
+    """The same table built by the device kernel the text session uses for its own copy (rope.zig:32-128)."""
+    ctx = ctx or default_context()
+    if end <= 0 or theta <= 0:
+        raise ValueError("EndTooSmall / ThetaTooSmall")
+    buf = ctx.alloc(max(1, (dim // 2) * end * 2 * 4))
+    ctx.check(ctx.lib.moon_dev_rope_table(ctx.handle, buf.ptr, dim, end, theta))
+    ctx.sync()
+    out = buf.to_host((end, dim // 2, 2), dtype=np.float32)
+    buf.free()
+    return out
+
+
 def apply_rot_emb(x, n_heads: int, head_dim: int, freqs_cis: np.ndarray, position_ids, rot_dim: int,
                   ctx: Context | None = None) -> np.ndarray:
     """applyRotEmb (rope.zig:130-272): x [n_heads, seq_len, head_dim]."""

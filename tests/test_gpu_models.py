@@ -306,3 +306,39 @@ def test_greedy_argmax_rules_in_every_mode(moon, O, ctx, case):
         assert dev.greedy(3).tolist() == [want] * 3, (case, mode)
         assert dev.position == 5 + 3
     dev.close()
+
+
+def test_session_recovers_after_a_failed_wait(moon, O, ctx):
+    """The error word of the fused decode kernels raised from the host (every kernel still runs to its end; a workgroup that
+    has to poll for long leaves early, as after an expired wait): the call fails with HipError, the session refuses work
+    until reset, and after reset it decodes exactly like a fresh session."""
+    dev = moon.text_model.TextModel(moon.text_model.default_config(), seed=0, std=0.02, ctx=ctx)
+    ids = O.fill_uniform_u32(64, 0, 50, 51200)
+    dev.forward(ids)
+    want = dev.greedy(6).tolist()
+    want_logits = dev.logits().copy()
+    dev.reset()
+    dev.forward(ids)
+    ctx.check(ctx.lib.moon_text_debug_raise_wait_error(dev.handle))
+    with pytest.raises(moon.context.HipError):
+        dev.greedy(3)
+    with pytest.raises(moon.context.HipError):
+        dev.greedy(1)  # refused until reset
+    with pytest.raises(moon.context.HipError):
+        dev.forward(ids[:2])
+    dev.reset()
+    assert dev.position == 0
+    dev.forward(ids)
+    assert dev.greedy(6).tolist() == want
+    assert np.array_equal(dev.logits().view(np.uint16), want_logits.view(np.uint16))
+    # and once more through the two-kernel path, whose error word is raised by the same hook
+    dev.reset()
+    dev.set_decode_mode(3)
+    dev.forward(ids)
+    ctx.check(ctx.lib.moon_text_debug_raise_wait_error(dev.handle))
+    with pytest.raises(moon.context.HipError):
+        dev.greedy(2)
+    dev.reset()
+    dev.forward(ids)
+    assert dev.greedy(6).tolist() == want
+    dev.close()

@@ -102,3 +102,22 @@ def test_greedy_profile_advances_like_greedy(moon, ctx):
         assert [prof[k][1] for k in m.PROFILE_KERNELS] in counts  # modes 0 and 3 fold kernels together where the device allows
         assert all(us > 0 for us, n in prof.values() if n)
     m.close()
+
+
+def test_device_rope_table_matches_oracle(moon, O, ctx):
+    """rope.precomputeFreqsCis (rope.zig:32-128) as the device builds it for the text session: all 2048 x 16 x 2 entries
+    against the oracle's table.  Both evaluate the reference's f32 steps; pow, cos and sin come from different libraries, each
+    within an ulp or two of the true value, and the entries are in [-1, 1]: the bound is 2 ulp of 1.0 in absolute terms."""
+    want = O.rope_table(32, 2048, 10000.0)
+    got = moon.rope.precompute_freqs_cis_device(32, 2048, 10000.0, ctx=ctx)
+    assert got.shape == want.shape == (2048, 16, 2)
+    diff = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    print(f"device rope table: max |diff| {diff.max():.3e}, entries that differ {int((diff > 0).sum())} of {diff.size}")
+    assert diff.max() <= 2.0 ** -22
+    assert np.array_equal(got[0], want[0])  # position 0: cos 1, sin 0 exactly
+    # a smaller table with another base
+    want = O.rope_table(8, 33, 500.0)
+    got = moon.rope.precompute_freqs_cis_device(8, 33, 500.0, ctx=ctx)
+    assert np.abs(got.astype(np.float64) - want).max() <= 2.0 ** -22
+    with pytest.raises(moon.context.InvalidRotationDimension):
+        moon.rope.precompute_freqs_cis_device(7, 4, ctx=ctx)
