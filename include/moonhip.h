@@ -202,6 +202,14 @@ int moon_dev_sdpa(moon_ctx *ctx, const void *q, const void *k, const void *v, vo
  * (q | k | v, text_model.zig:198-226); out is [n_heads*head_dim] (already head-merged, :293-294). */
 int moon_dev_decode_attention(moon_ctx *ctx, const void *qkv, void *cache_k, void *cache_v, const void *freqs_cis,
                               void *out, size_t n_heads, size_t head_dim, size_t rot_dim, size_t max_seq, size_t pos);
+/* moon_dev_decode_attention for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and the same
+ * result bits; the split-KV partials live in a static device array of the library (270,336 bytes per device, held until
+ * the process ends) instead of a workspace grown on demand, so the call performs no hipMalloc / hipFree.  n_heads above
+ * 128 -> MOON_EINVAL_DIM.  All calls on one device share that array: calls that overlap on one device (two contexts, two
+ * threads) race; calls on one context are serialised as always.  Asynchronous on the context's stream. */
+int moon_dev_decode_attention_noalloc(moon_ctx *ctx, const void *qkv, void *cache_k, void *cache_v, const void *freqs_cis,
+                                      void *out, size_t n_heads, size_t head_dim, size_t rot_dim, size_t max_seq, size_t pos);
 /* rope.precomputeFreqsCis(f32, dim, end, theta) (rope.zig:32-128) on the device: table[end, rot_dim/2, 2] f32 of
  * (cos, sin)(p * theta^(-2i/rot_dim)), the table the text session builds for itself (text_model.zig:88) and
  * moon_dev_decode_attention reads.  rot_dim odd or zero -> MOON_EROT_DIM. */

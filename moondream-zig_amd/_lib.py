@@ -102,6 +102,7 @@ SIGNATURES = {
     "moon_dev_linear": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _i, _vp, _i, _vp]),
     "moon_dev_sdpa": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _l, _vp, _sz]),
     "moon_dev_decode_attention": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]),
+    "moon_dev_decode_attention_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz]),
     "moon_dev_rope_table": (_i, [_vp, _vp, _sz, _sz, _f]),
     "moon_dev_layernorm": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _f]),
     "moon_timer_start": (_i, [_vp]),

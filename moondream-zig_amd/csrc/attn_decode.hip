@@ -9,6 +9,7 @@
 // un-normalised partial (o, m, l) in f32; a second kernel merges the partials in a fixed order.
 // The cache is read in place in the reference layout [n_heads][max_seq][head_dim]; no "active" copy is made.
 #include "attn_decode.hpp"
+#include <mutex>
 
 namespace {
 
@@ -59,6 +60,58 @@ int launch_decode_attention_plain(moon_ctx *ctx, const half_t *q, const half_t *
                        (int)kv_len - 1, (const uint32_t *)nullptr);
     MOON_HIP(ctx, hipGetLastError());
     hipLaunchKernelGGL(decode_attn_merge_kernel<64>, dim3((unsigned)H), dim3(64), 0, ctx->stream, partial, out);
+    MOON_HIP(ctx, hipGetLastError());
+    return MOON_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same step for callers that cannot allocate device memory (code under HIP graph capture, serving loops, harnesses
+// that forbid hipMalloc): the split partials live in a file-scope device array instead of the context's grown workspace.
+// Every device the library runs on holds its own copy of the array (MOON_NOALLOC_MAX_HEADS * DEC_SPLITS * 66 floats =
+// 270,336 bytes) until the process ends.  In host code the array's name is only a handle: the device address is asked
+// for once per device (decode_attention_static_init, called with that device current when a context is created) and
+// only that address is ever handed to a kernel.  Every launch writes all partials of its n_heads before its merge
+// kernel reads them (a split without keys writes m = -inf, l = 0, o = 0), so nothing of an earlier call is read and
+// nothing needs clearing; two calls that overlap on one device (different contexts or streams) race on the array.
+constexpr size_t MOON_NOALLOC_MAX_HEADS = 128;
+constexpr int MOON_NOALLOC_MAX_DEVICES = 64;
+static __device__ __align__(256) float scratch[MOON_NOALLOC_MAX_HEADS * DEC_SPLITS * (64 + 2)];
+static float *g_scratch_ptr[MOON_NOALLOC_MAX_DEVICES]; // device address of `scratch` on each device, null until asked for
+static std::mutex g_scratch_mu;
+
+int decode_attention_static_init(moon_ctx *ctx) {
+    if (ctx->device < 0 || ctx->device >= MOON_NOALLOC_MAX_DEVICES) return MOON_OK; // the no-alloc entry point reports it
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[ctx->device]) return MOON_OK;
+    float *p = nullptr;
+    MOON_HIP(ctx, hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch))); // the current device's copy
+    g_scratch_ptr[ctx->device] = p;
+    return MOON_OK;
+}
+
+extern "C" int moon_dev_decode_attention_noalloc(moon_ctx *ctx, const void *qkv, void *cache_k, void *cache_v, const void *freqs_cis,
+                                                 void *out, size_t n_heads, size_t head_dim, size_t rot_dim, size_t max_seq, size_t pos) {
+    if (!ctx) return MOON_EINVAL;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (!qkv || !cache_k || !cache_v || !freqs_cis || !out) return moon_fail(ctx, MOON_EINVAL, "dev_decode_attention_noalloc: null operand");
+    if (head_dim != 64) return moon_fail(ctx, MOON_EINVAL_DIM, "decode attention: head_dim %zu unsupported (64 only)", head_dim);
+    if (!n_heads || n_heads > MOON_NOALLOC_MAX_HEADS)
+        return moon_fail(ctx, MOON_EINVAL_DIM, "dev_decode_attention_noalloc: n_heads %zu outside 1..%zu (the static workspace holds %zu heads)",
+                         n_heads, MOON_NOALLOC_MAX_HEADS, MOON_NOALLOC_MAX_HEADS);
+    if (rot_dim > head_dim || rot_dim % 2) return moon_fail(ctx, MOON_EROT_DIM, "decode attention: bad rot_dim %zu", rot_dim);
+    if (max_seq > 2048 || pos >= max_seq)
+        return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "decode attention: pos %zu >= max_seq %zu (limit 2048)", pos, max_seq);
+    float *partial = nullptr;
+    if (ctx->device >= 0 && ctx->device < MOON_NOALLOC_MAX_DEVICES) {
+        std::lock_guard<std::mutex> slock(g_scratch_mu);
+        partial = g_scratch_ptr[ctx->device];
+    }
+    if (!partial) return moon_fail(ctx, MOON_EHIP, "dev_decode_attention_noalloc: no static workspace on device %d", ctx->device);
+    hipLaunchKernelGGL((decode_attn_partial_kernel<64, true>), dim3((unsigned)(n_heads * DEC_SPLITS)), dim3(256), 0, ctx->stream,
+                       (const half_t *)qkv, (half_t *)cache_k, (half_t *)cache_v, (const float *)freqs_cis, partial, (int)n_heads,
+                       (int)rot_dim, (int)max_seq, (int)pos, (const uint32_t *)nullptr);
+    MOON_HIP(ctx, hipGetLastError());
+    hipLaunchKernelGGL(decode_attn_merge_kernel<64>, dim3((unsigned)n_heads), dim3(64), 0, ctx->stream, partial, (half_t *)out);
     MOON_HIP(ctx, hipGetLastError());
     return MOON_OK;
 }

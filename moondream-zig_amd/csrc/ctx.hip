@@ -57,6 +57,11 @@ extern "C" int moon_ctx_create(int device, moon_ctx **out) {
         delete ctx;
         return rc;
     }
+    if (int rc = decode_attention_static_init(ctx); rc != MOON_OK) { // the device is current here
+        g_create_error = ctx->err;
+        moon_ctx_destroy(ctx);
+        return rc;
+    }
     *out = ctx;
     return MOON_OK;
 }

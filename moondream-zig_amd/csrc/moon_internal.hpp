@@ -111,6 +111,8 @@ int launch_sdpa(moon_ctx *ctx, const half_t *q, const half_t *k, const half_t *v
 int launch_decode_attention(moon_ctx *ctx, const half_t *qkv, half_t *cache_k, half_t *cache_v, const float *table,
                             half_t *out, size_t H, size_t D, size_t rot_dim, size_t max_seq, size_t pos,
                             const uint32_t *pos_dev);
+// asks for the device address of the static workspace of moon_dev_decode_attention_noalloc on ctx->device (once per device)
+int decode_attention_static_init(moon_ctx *ctx);
 int launch_sdpa_generic(moon_ctx *ctx, const half_t *q, const half_t *k, const half_t *v, half_t *out, size_t H, size_t Lq,
                         size_t Lkv, size_t D, size_t kv_head_stride, long causal_pos, const uint8_t *mask, size_t mask_stride,
                         bool out_merged);
