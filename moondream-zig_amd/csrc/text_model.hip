@@ -5,6 +5,7 @@
 // Activations and the cache never leave the device; a decode step enqueues kernels only (token id and position
 // are read from device memory), so the loop needs no host synchronisation until the ids are fetched.
 #include "moon_internal.hpp"
+#include "decode_stream.hpp"
 
 #include <cstdlib>
 #include <algorithm>
@@ -113,6 +114,14 @@ struct moon_text_model {
     std::vector<uint32_t> layer_launches;
     uint32_t *lm_exchange = nullptr;  // arg-max pairs of the LM head's workgroups, then their counter (monotonic)
     uint32_t lm_launches = 0;
+    // streaming decode kernel (decode mode 4): the whole greedy loop as one launch, decode_stream.hip
+    bool stream = false;              // shape and device supported
+    half_t *fc2_wt = nullptr, *out_wt = nullptr; // [L][ffn][d], [L][d][d]: transposed copies made at creation
+    half_t *stream_arena = nullptr;   // one allocation holding qkv_w, fc1_w, fc2_wt, out_wt, lin_w (the kernel addresses them with 32-bit offsets)
+    size_t stream_arena_bytes = 0;
+    uint32_t *stream_sync = nullptr;  // hid_t | qkv_t | ap_t | rp_t | am_t | error word, see stream_layout()
+    uint32_t stream_gen = 0;          // tags used so far on those buffers
+    long long *stream_trace = nullptr;
     long long *layer_trace = nullptr; // [grid][8] stamps of the most recent layer launch when MOON_DECODE_TRACE is set
     struct StepProfiler *prof = nullptr;  // set only inside moon_text_greedy_profile
     std::vector<void *> allocs;
@@ -155,20 +164,48 @@ int check_cfg(moon_ctx *ctx, const moon_text_config *c) {
     return MOON_OK;
 }
 
+// 32-bit word offsets of the streaming kernel's exchange buffers inside stream_sync (the 64-bit ones on 8-byte boundaries)
+struct StreamLayout {
+    size_t hid, qkv, ap, rp, rp_flag, am, err, words;
+};
+StreamLayout stream_layout() {
+    StreamLayout o;
+    o.hid = 0;
+    o.qkv = o.hid + STREAM_HID_WORDS;
+    o.ap = o.qkv + STREAM_QKV_WORDS;
+    o.rp = o.ap + 2 * STREAM_AP_WORDS;
+    o.rp_flag = o.rp + STREAM_RP_FLOATS;
+    o.am = o.rp_flag + STREAM_RP_FLAGS;
+    o.err = o.am + 2 * STREAM_AM_WORDS + 32; // a line of its own
+    o.words = o.err + 32;
+    return o;
+}
+
 int alloc_all(moon_text_model *m) {
     const Sizes z = sizes(m->cfg);
+    m->stream = decode_stream_supported(m->ctx, z.d, z.ffn, z.H, z.D, z.S, z.L, z.V);
+    if (m->stream) { // the matrices the streaming kernel reads, in one allocation
+        const size_t n_qkv = z.L * 3 * z.d * z.d, n_fc = z.L * z.ffn * z.d, n_out = z.L * z.d * z.d, n_lin = z.V * z.d;
+        m->stream_arena_bytes = (n_qkv + 2 * n_fc + n_out + n_lin) * sizeof(half_t);
+        MOON_TRY(dalloc_t(m, n_qkv + 2 * n_fc + n_out + n_lin, &m->stream_arena));
+        m->qkv_w = m->stream_arena;
+        m->fc1_w = m->qkv_w + n_qkv;
+        m->fc2_wt = m->fc1_w + n_fc;
+        m->out_wt = m->fc2_wt + n_fc;
+        m->lin_w = m->out_wt + n_out;
+    }
     MOON_TRY(dalloc_t(m, z.V * z.d, &m->wte));
     MOON_TRY(dalloc_t(m, z.L * z.d, &m->ln_w));
     MOON_TRY(dalloc_t(m, z.L * z.d, &m->ln_b));
-    MOON_TRY(dalloc_t(m, z.L * 3 * z.d * z.d, &m->qkv_w));
+    if (!m->stream) MOON_TRY(dalloc_t(m, z.L * 3 * z.d * z.d, &m->qkv_w));
     MOON_TRY(dalloc_t(m, z.L * 3 * z.d, &m->qkv_b));
     MOON_TRY(dalloc_t(m, z.L * z.d * z.d, &m->out_w));
     MOON_TRY(dalloc_t(m, z.L * z.d, &m->out_b));
-    MOON_TRY(dalloc_t(m, z.L * z.ffn * z.d, &m->fc1_w));
+    if (!m->stream) MOON_TRY(dalloc_t(m, z.L * z.ffn * z.d, &m->fc1_w));
     MOON_TRY(dalloc_t(m, z.L * z.ffn, &m->fc1_b));
     MOON_TRY(dalloc_t(m, z.L * z.d * z.ffn, &m->fc2_w));
     MOON_TRY(dalloc_t(m, z.L * z.d, &m->fc2_b));
-    MOON_TRY(dalloc_t(m, z.V * z.d, &m->lin_w));
+    if (!m->stream) MOON_TRY(dalloc_t(m, z.V * z.d, &m->lin_w));
     MOON_TRY(dalloc_t(m, z.V, &m->lin_b));
     MOON_TRY(dalloc_t(m, z.d, &m->lno_w));
     MOON_TRY(dalloc_t(m, z.d, &m->lno_b));
@@ -211,7 +248,16 @@ int alloc_all(moon_text_model *m) {
     m->layer_launches.assign(z.L, 0);
     MOON_TRY(dalloc_t(m, decode_lm_head_words(m->ctx), &m->lm_exchange));
     MOON_TRY(launch_fill_uniform_u32(m->ctx, m->lm_exchange, decode_lm_head_words(m->ctx), 0, 0, 1)); // zeros
+    if (m->stream) {
+        MOON_TRY(dalloc_t(m, stream_layout().words, &m->stream_sync));
+        MOON_TRY(launch_fill_uniform_u32(m->ctx, m->stream_sync, stream_layout().words, 0, 0, 1)); // zeros
+        m->decode_mode = 4;
+    }
     if (getenv("MOON_DECODE_TRACE")) {
+        if (m->stream) {
+            MOON_TRY(dalloc_t(m, z.L * size_t(STREAM_GRID) * 8, &m->stream_trace));
+            MOON_TRY(launch_fill_uniform_u32(m->ctx, (uint32_t *)m->stream_trace, z.L * size_t(STREAM_GRID) * 16, 0, 0, 1));
+        }
         MOON_TRY(dalloc_t(m, size_t(4096) * 8, &m->layer_trace));
         MOON_TRY(launch_fill_uniform_u32(m->ctx, (uint32_t *)m->layer_trace, size_t(4096) * 16, 0, 0, 1));
     }
@@ -240,10 +286,23 @@ int clear_sync_state(moon_text_model *m) {
     MOON_TRY(launch_fill_uniform_u32(ctx, m->front_sync, z.L * z.H * 32 + 1, 0, 0, 1));
     MOON_TRY(launch_fill_uniform_u32(ctx, m->layer_sync, z.L * m->layer_sync_words + 1, 0, 0, 1));
     MOON_TRY(launch_fill_uniform_u32(ctx, m->lm_exchange, decode_lm_head_words(ctx), 0, 0, 1));
+    if (m->stream) MOON_TRY(launch_fill_uniform_u32(ctx, m->stream_sync, stream_layout().words, 0, 0, 1));
+    m->stream_gen = 0;
     m->attn_launches.assign(z.L, 0);
     m->front_launches.assign(z.L, 0);
     m->layer_launches.assign(z.L, 0);
     m->lm_launches = 0;
+    return MOON_OK;
+}
+
+// The streaming kernel reads fc2 and out_proj by input column: transposed copies, made once when the weights are in place.
+int prepare_stream(moon_text_model *m) {
+    if (!m->stream) return MOON_OK;
+    const Sizes z = sizes(m->cfg);
+    for (size_t l = 0; l < z.L; l++) {
+        MOON_TRY(launch_transpose(m->ctx, m->fc2_w + l * z.d * z.ffn, m->fc2_wt + l * z.ffn * z.d, z.d, z.ffn));
+        MOON_TRY(launch_transpose(m->ctx, m->out_w + l * z.d * z.d, m->out_wt + l * z.d * z.d, z.d, z.d));
+    }
     return MOON_OK;
 }
 
@@ -281,7 +340,8 @@ int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool p
     if (n == 1 && m->fused) {
         // three kernels: LN + qkv + fc1;  rope + append + attention (+ merge);  out_proj + fc2 + both residual adds
         const half_t *x = token_dev ? m->wte : m->hidden;
-        if (m->whole_layer && m->decode_mode == 0) {
+        const int mode = m->decode_mode == 4 ? 0 : m->decode_mode; // the streaming kernel is a loop; single steps take the per-layer kernels
+        if (m->whole_layer && mode == 0) {
             // one kernel for the layer
             const uint32_t head_target = ++m->attn_launches[layer] * 8u;
             const uint32_t generation = ++m->layer_launches[layer];
@@ -292,7 +352,7 @@ int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool p
                                        m->layer_sync + z.L * m->layer_sync_words, z.H, m->cfg.rot_dim, z.S, pos,
                                        pos_on_device ? m->state_dev : nullptr, m->layer_trace);
         }
-        if (m->front && (m->decode_mode == 0 || m->decode_mode == 3)) {
+        if (m->front && (mode == 0 || mode == 3)) {
             // two kernels: LN + qkv + fc1 with the attention hidden under the fc1 stream;  out_proj + fc2 + residual adds
             const uint32_t head_target = ++m->attn_launches[layer] * 8u;
             const uint32_t qkv_target = ++m->front_launches[layer] * (uint32_t)(3 * z.D);
@@ -403,6 +463,7 @@ extern "C" int moon_text_model_create(moon_ctx *ctx, const moon_text_config *cfg
     up(m->lin_b, w->t_linear_b, z.V);
     up(m->lno_w, w->t_ln_out_w, z.d);
     up(m->lno_b, w->t_ln_out_b, z.d);
+    if (rc == MOON_OK) rc = prepare_stream(m);
     if (rc == MOON_OK) {
         hipError_t e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) rc = moon_fail(ctx, MOON_EHIP, "weight upload sync: %s", hipGetErrorString(e));
@@ -450,6 +511,7 @@ extern "C" int moon_text_model_create_synthetic(moon_ctx *ctx, const moon_text_c
     rnd(m->lin_b, z.V, 12);
     cst(m->lno_w, z.d, 1.0f);
     cst(m->lno_b, z.d, 0.0f);
+    if (rc == MOON_OK) rc = prepare_stream(m);
     if (rc == MOON_OK) {
         hipError_t e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) rc = moon_fail(ctx, MOON_EHIP, "synthetic weights: %s", hipGetErrorString(e));
@@ -565,6 +627,34 @@ static void print_layer_trace(moon_text_model *m) {
     }
 }
 
+// MOON_DECODE_TRACE with the streaming kernel: per layer of the last step, when the workgroups passed the kernel's eight
+// stamps (microseconds after the layer's first workgroup started it; mean and latest over the 256 workgroups)
+static void print_stream_trace(moon_text_model *m) {
+    const Sizes z = sizes(m->cfg);
+    std::vector<long long> t(z.L * size_t(STREAM_GRID) * 8);
+    if (hipMemcpy(t.data(), m->stream_trace, t.size() * sizeof(long long), hipMemcpyDeviceToHost) != hipSuccess) return;
+    const char *names[8] = {"start", "hidden in", "qkv out", "3 fc pairs", "attn partial out", "head merged", "partials out", "hidden out"};
+    long long t_first = t[0];
+    for (size_t b = 0; b < STREAM_GRID; b++) t_first = std::min(t_first, t[b * 8]);
+    fprintf(stderr, "[moonhip stream trace] last step, per layer: stamp mean/max us after the layer's first start; layer start after step's first layer start\n");
+    for (size_t l = 0; l < z.L; l++) {
+        const long long *tl = t.data() + l * STREAM_GRID * 8;
+        long long t0 = tl[0];
+        for (size_t b = 0; b < STREAM_GRID; b++) t0 = std::min(t0, tl[b * 8]);
+        fprintf(stderr, "  layer %2zu (+%7.1f):", l, (double)(t0 - t_first) * 0.01);
+        for (int i = 1; i < 8; i++) {
+            double sum = 0, mx = 0;
+            for (size_t b = 0; b < STREAM_GRID; b++) {
+                const double us = (double)(tl[b * 8 + i] - t0) * 0.01;
+                sum += us;
+                mx = std::max(mx, us);
+            }
+            fprintf(stderr, " %s %.1f/%.1f", names[i], sum / STREAM_GRID, mx);
+        }
+        fprintf(stderr, "\n");
+    }
+}
+
 // sampling == nullptr: greedy.  Otherwise sampling.sample with u[step] in place of the arg-max (the per-launch kernels only).
 static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, const moon_sampling_config *sampling = nullptr,
                          const float *u = nullptr) {
@@ -577,6 +667,52 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
         return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "text_greedy: %zu + %zu tokens > max_seq %zu (SequenceTooLong)", m->cur_len, n_steps, m->cfg.max_seq);
     MOON_HIP(ctx, hipSetDevice(ctx->device));
     if (sampling) MOON_HIP(ctx, hipMemcpyAsync(m->u_dev, u, n_steps * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    if (!sampling && m->decode_mode == 4 && m->stream && !m->prof) {
+        const Sizes z = sizes(m->cfg);
+        const StreamLayout lay = stream_layout();
+        if ((uint64_t)m->stream_gen + (uint64_t)n_steps * z.L + 2 > 0xfffffff0ull) { // tags count up for the life of the session
+            MOON_TRY(launch_fill_uniform_u32(ctx, m->stream_sync, lay.words, 0, 0, 1));
+            m->stream_gen = 0;
+        }
+        StreamParams p;
+        p.wte = m->wte; p.ln_w = m->ln_w; p.ln_b = m->ln_b; p.qkv_b = m->qkv_b; p.fc1_b = m->fc1_b;
+        p.fc2_b = m->fc2_b; p.out_b = m->out_b; p.lin_b = m->lin_b; p.lno_w = m->lno_w; p.lno_b = m->lno_b;
+        p.w_base = m->stream_arena; p.w_bytes = m->stream_arena_bytes;
+        p.off_qkv = (uint32_t)((m->qkv_w - m->stream_arena) * sizeof(half_t)); p.off_fc1 = (uint32_t)((m->fc1_w - m->stream_arena) * sizeof(half_t));
+        p.off_fc2t = (uint32_t)((m->fc2_wt - m->stream_arena) * sizeof(half_t)); p.off_outt = (uint32_t)((m->out_wt - m->stream_arena) * sizeof(half_t));
+        p.off_lin = (uint32_t)((m->lin_w - m->stream_arena) * sizeof(half_t));
+        p.cache_k = m->cache_k; p.cache_v = m->cache_v; p.freqs = m->freqs;
+        p.hidden_first = m->hidden + (m->last_n - 1) * z.d; p.hidden_out = m->hidden; p.logits = m->logits;
+        p.hid_t = m->stream_sync + lay.hid; p.qkv_t = m->stream_sync + lay.qkv;
+        p.ap_t = reinterpret_cast<unsigned long long *>(m->stream_sync + lay.ap);
+        p.rp = reinterpret_cast<float *>(m->stream_sync + lay.rp);
+        p.rp_flag = m->stream_sync + lay.rp_flag;
+        p.am_t = reinterpret_cast<unsigned long long *>(m->stream_sync + lay.am);
+        p.error = m->stream_sync + lay.err;
+        p.out_ids = m->ids_dev;
+        p.L = (int)z.L; p.V = (int)z.V; p.rot_dim = (int)m->cfg.rot_dim; p.max_seq = (int)z.S; p.pos0 = (int)m->cur_len; p.n_steps = (int)n_steps;
+        p.eps = m->cfg.ln_eps; p.gen0 = m->stream_gen;
+        p.timeout_ticks = getenv("MOON_STREAM_NOWAIT") ? -1 : 100000000LL; // 1 s of the 100 MHz wall clock
+        p.trace = m->stream_trace;
+        MOON_TRY(launch_decode_stream(ctx, p));
+        m->stream_gen += (uint32_t)(n_steps * z.L);
+        uint32_t error_flag = 0;
+        MOON_HIP(ctx, hipMemcpyAsync(out_ids, m->ids_dev, n_steps * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+        MOON_HIP(ctx, hipMemcpyAsync(&error_flag, p.error, sizeof(error_flag), hipMemcpyDeviceToHost, ctx->stream));
+        MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        if (error_flag != 0) {
+            m->cache_invalid = true;
+            m->last_n = 0;
+            (void)clear_sync_state(m);
+            return moon_fail(ctx, MOON_EHIP, "streaming decode kernel: a wait between workgroups timed out; the session needs moon_text_reset");
+        }
+        if (m->stream_trace) print_stream_trace(m);
+        m->cur_len += n_steps;
+        m->last_n = 1;
+        hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->state_dev, (uint32_t)m->cur_len, 0u);
+        MOON_HIP(ctx, hipGetLastError());
+        return MOON_OK;
+    }
     if (!sampling && m->decode_mode == 1 && m->groups > 0) {
         const Sizes z = sizes(m->cfg);
         DecodeParams p;
@@ -630,7 +766,8 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
     uint32_t *state = m->state_dev;
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, state, (uint32_t)m->cur_len, 0u);
     MOON_HIP(ctx, hipGetLastError());
-    const bool use_layer = m->whole_layer && m->decode_mode == 0;
+    const int mode = m->decode_mode == 4 ? 0 : m->decode_mode; // sampled decoding and profiled steps take the per-layer kernels
+    const bool use_layer = m->whole_layer && mode == 0;
     if (use_layer) { // counters count up for the life of the model: clear them long before 32 bits are used up (192 per launch)
         const Sizes z = sizes(m->cfg);
         if ((uint64_t(m->layer_launches[0]) + n_steps + 1) * 192ull > 0x7fffffffull) {
@@ -638,7 +775,7 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
             m->layer_launches.assign(z.L, 0);
         }
     }
-    const bool use_front = !use_layer && m->front && (m->decode_mode == 0 || m->decode_mode == 3);
+    const bool use_front = !use_layer && m->front && (mode == 0 || mode == 3);
     if (use_front) { // the row counters count up for the life of the model: clear them long before 32 bits are used up
         const Sizes z = sizes(m->cfg);
         const uint64_t per_launch = 3 * z.D;
@@ -765,15 +902,21 @@ extern "C" int moon_text_debug_raise_wait_error(moon_text_model *m) {
     MOON_HIP(ctx, hipGetLastError());
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->front_sync + z.L * z.H * 32 - 1, 0u, 1u);
     MOON_HIP(ctx, hipGetLastError());
+    if (m->stream) { // the error word sits in a line of its own: {0, 1} to (the unused word before it, the error word)
+        hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->stream_sync + stream_layout().err - 1, 0u, 1u);
+        MOON_HIP(ctx, hipGetLastError());
+    }
     return MOON_OK;
 }
 
 extern "C" int moon_text_set_decode_mode(moon_text_model *m, int mode) {
     if (!m) return MOON_EINVAL;
     std::lock_guard<std::mutex> lock(m->ctx->mu);
-    if (mode < 0 || mode > 3)
+    if (mode < 0 || mode > 4)
         return moon_fail(m->ctx, MOON_EINVAL,
-                         "decode mode must be 0 (one kernel per layer), 1 (persistent kernel), 2 (three kernels per layer) or 3 (two kernels per layer)");
+                         "decode mode must be 0 (one kernel per layer), 1 (persistent kernel with barriers), 2 (three kernels per layer), 3 (two kernels per "
+                         "layer) or 4 (streaming kernel)");
+    if (mode == 4 && !m->stream) return moon_fail(m->ctx, MOON_EINVAL, "streaming decode kernel unavailable for this configuration or device");
     if (mode == 1 && m->groups == 0) return moon_fail(m->ctx, MOON_EINVAL, "persistent decode kernel unavailable for this configuration");
     m->decode_mode = mode;
     return MOON_OK;
