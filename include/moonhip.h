@@ -280,8 +280,12 @@ int moon_text_greedy_profile(moon_text_model *m, size_t n_steps, uint32_t *out_i
  * attention output to each other through counters, with bounded waits) where the device can hold enough of that
  * kernel's workgroups at once, else as mode 3 or 2; 1 = one persistent kernel for the whole greedy loop (all workgroups
  * co-resident, device-wide barriers between phases); 2 = three kernels per layer and no waits inside kernels;
- * 3 = two kernels per layer (LayerNorm + qkv + fc1 + attention; out_proj + fc2 + residual).  All produce the same bits.
- * A wait that expires makes the call return MOON_EHIP. */
+ * 3 = two kernels per layer (LayerNorm + qkv + fc1 + attention; out_proj + fc2 + residual).  Modes 0-3 produce the same bits.
+ * 4 = the streaming kernel: the whole greedy loop as one launch that keeps every compute unit reading weights through LDS
+ * rings while two workgroups per unit exchange q/k/v, attention partials, partial sums of out_proj / fc2 and the hidden
+ * state through tagged words (default configuration on a 256-unit device only; out_proj and fc2 are summed per workgroup and
+ * then over workgroups, so its logits differ from the other modes' in the last bits: same tolerance, same token ids in
+ * the tests).  A wait that expires makes the call return MOON_EHIP. */
 int moon_text_set_decode_mode(moon_text_model *m, int mode);
 /* After a MOON_EHIP from moon_text_greedy / moon_text_sample caused by an expired wait inside a fused decode kernel the
  * session refuses further forward / greedy / sample calls until moon_text_reset: workgroups that gave up may have skipped

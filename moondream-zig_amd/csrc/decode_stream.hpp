@@ -20,22 +20,23 @@ struct StreamParams {
     uint32_t *hid_t;            // [d]      f16 bits | tag16 << 16 : hidden state after a layer
     uint32_t *qkv_t;            // [3d]     f16 bits | tag16 << 16 : q | k | v of the new token
     unsigned long long *ap_t;   // [H][8][66]       f32 bits | tag << 32 : attention partials (o[64], m, l) per (head, split)
-    float *rp;                  // [256 sources][256 slots][16] f32: partial sums of fc2 (0-7) and out_proj (8-15) for a reducer
-    uint32_t *rp_flag;          // [256 sources][4 wavefronts]: tag of the layer-step whose partial sums are complete
-    unsigned long long *am_t;   // [256]   f16 bits | tag16 << 16 | index << 32 : arg-max pair of a workgroup
+    float *rp;                  // [2 kinds: fc2, out_proj][256 source units][256 slots][8] f32: partial sums for a reducer
+    uint32_t *rp_flag;          // [2 kinds][256 source units][8 wavefronts]: tag of the layer-step whose partial sums are complete
+    unsigned long long *am_t;   // [512]   f16 bits | tag16 << 16 | index << 32 : arg-max pair of a workgroup
     uint32_t *error;            // raised when a wait expires; every wait ends when it is up
     uint32_t *out_ids;          // [n_steps]
     int L, V, rot_dim, max_seq, pos0, n_steps;
     float eps;
     uint32_t gen0;              // tags used by earlier launches on these buffers
     long long timeout_ticks;    // bound of every wait, 100 MHz ticks
-    long long *trace;           // optional [L][256][8] stamps of the last step (tuning aid), or null
+    int debug;                  // tuning builds only: bit 0 = the MLP workgroups stream nothing (wrong results)
+    long long *trace;           // optional [L][512][8] stamps of the last step (tuning aid), or null
 };
 
-constexpr int STREAM_GRID = 256, STREAM_THREADS = 256;
+constexpr int STREAM_GRID = 512, STREAM_THREADS = 512;
 constexpr int STREAM_D = 2048, STREAM_FFN = 8192, STREAM_H = 32, STREAM_HD = 64;
 constexpr size_t STREAM_HID_WORDS = STREAM_D, STREAM_QKV_WORDS = 3 * STREAM_D;
-constexpr size_t STREAM_AP_WORDS = size_t(STREAM_H) * 8 * 66, STREAM_RP_FLOATS = size_t(256) * 256 * 16, STREAM_RP_FLAGS = 256 * 4, STREAM_AM_WORDS = 256;
+constexpr size_t STREAM_AP_WORDS = size_t(STREAM_H) * 8 * 66, STREAM_RP_FLOATS = size_t(2) * 256 * 256 * 8, STREAM_RP_FLAGS = 2 * 256 * 8, STREAM_AM_WORDS = 512;
 
 bool decode_stream_supported(moon_ctx *ctx, size_t d, size_t ffn, size_t H, size_t D, size_t max_seq, size_t L, size_t V);
 int launch_decode_stream(moon_ctx *ctx, const StreamParams &p);

@@ -251,7 +251,6 @@ int alloc_all(moon_text_model *m) {
     if (m->stream) {
         MOON_TRY(dalloc_t(m, stream_layout().words, &m->stream_sync));
         MOON_TRY(launch_fill_uniform_u32(m->ctx, m->stream_sync, stream_layout().words, 0, 0, 1)); // zeros
-        m->decode_mode = 4;
     }
     if (getenv("MOON_DECODE_TRACE")) {
         if (m->stream) {
@@ -633,23 +632,35 @@ static void print_stream_trace(moon_text_model *m) {
     const Sizes z = sizes(m->cfg);
     std::vector<long long> t(z.L * size_t(STREAM_GRID) * 8);
     if (hipMemcpy(t.data(), m->stream_trace, t.size() * sizeof(long long), hipMemcpyDeviceToHost) != hipSuccess) return;
-    const char *names[8] = {"start", "hidden in", "qkv out", "3 fc pairs", "attn partial out", "head merged", "partials out", "hidden out"};
+    const char *names[8] = {"start", "hidden in", "qkv out", "q,k,v in", "attn partial out", "head merged", "partials out", "hidden out"};
     long long t_first = t[0];
     for (size_t b = 0; b < STREAM_GRID; b++) t_first = std::min(t_first, t[b * 8]);
     fprintf(stderr, "[moonhip stream trace] last step, per layer: stamp mean/max us after the layer's first start; layer start after step's first layer start\n");
     for (size_t l = 0; l < z.L; l++) {
         const long long *tl = t.data() + l * STREAM_GRID * 8;
         long long t0 = tl[0];
-        for (size_t b = 0; b < STREAM_GRID; b++) t0 = std::min(t0, tl[b * 8]);
-        fprintf(stderr, "  layer %2zu (+%7.1f):", l, (double)(t0 - t_first) * 0.01);
+        for (size_t b = 0; b < STREAM_GRID; b += 2) t0 = std::min(t0, tl[b * 8]);
+        fprintf(stderr, "  layer %2zu (+%7.1f) attention:", l, (double)(t0 - t_first) * 0.01);
         for (int i = 1; i < 8; i++) {
             double sum = 0, mx = 0;
-            for (size_t b = 0; b < STREAM_GRID; b++) {
+            for (size_t b = 0; b < STREAM_GRID; b += 2) {
                 const double us = (double)(tl[b * 8 + i] - t0) * 0.01;
                 sum += us;
                 mx = std::max(mx, us);
             }
-            fprintf(stderr, " %s %.1f/%.1f", names[i], sum / STREAM_GRID, mx);
+            fprintf(stderr, " %s %.1f/%.1f", names[i], sum / (STREAM_GRID / 2), mx);
+        }
+        fprintf(stderr, " | mlp:");
+        const int mlp_stamps[5] = {0, 1, 2, 3, 6};
+        const char *mlp_names[5] = {"start", "hidden in", "fc1 done", "fc2 done", "partials out"};
+        for (int k = 0; k < 5; k++) {
+            double sum = 0, mx = 0;
+            for (size_t b = 1; b < STREAM_GRID; b += 2) {
+                const double us = (double)(tl[b * 8 + mlp_stamps[k]] - t0) * 0.01;
+                sum += us;
+                mx = std::max(mx, us);
+            }
+            fprintf(stderr, " %s %.1f/%.1f", mlp_names[k], sum / (STREAM_GRID / 2), mx);
         }
         fprintf(stderr, "\n");
     }
@@ -694,6 +705,7 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
         p.eps = m->cfg.ln_eps; p.gen0 = m->stream_gen;
         p.timeout_ticks = getenv("MOON_STREAM_NOWAIT") ? -1 : 100000000LL; // 1 s of the 100 MHz wall clock
         p.trace = m->stream_trace;
+        p.debug = getenv("MOON_STREAM_DEBUG") ? atoi(getenv("MOON_STREAM_DEBUG")) : 0;
         MOON_TRY(launch_decode_stream(ctx, p));
         m->stream_gen += (uint32_t)(n_steps * z.L);
         uint32_t error_flag = 0;

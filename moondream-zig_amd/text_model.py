@@ -64,7 +64,8 @@ class TextModel:
         self.ctx.check(self.ctx.lib.moon_text_reset(self.handle))
 
     def set_decode_mode(self, mode: int):
-        """0 (default): two fused kernels per layer; 1: one persistent kernel for the greedy loop; 2: three kernels per layer."""
+        """0 (default): one fused kernel per layer; 1: one persistent kernel with device-wide barriers; 2: three kernels per
+        layer; 3: two per layer; 4: the streaming kernel (whole loop in one launch, tagged exchanges between workgroups)."""
         self.ctx.check(self.ctx.lib.moon_text_set_decode_mode(self.handle, mode))
 
     @property

@@ -331,14 +331,58 @@ def test_session_recovers_after_a_failed_wait(moon, O, ctx):
     dev.forward(ids)
     assert dev.greedy(6).tolist() == want
     assert np.array_equal(dev.logits().view(np.uint16), want_logits.view(np.uint16))
-    # and once more through the two-kernel path, whose error word is raised by the same hook
-    dev.reset()
-    dev.set_decode_mode(3)
+    # and once more through the two-kernel path and the streaming kernel, whose error words are raised by the same hook
+    for mode in (3, 4):
+        dev.reset()
+        dev.set_decode_mode(mode)
+        dev.forward(ids)
+        ctx.check(ctx.lib.moon_text_debug_raise_wait_error(dev.handle))
+        with pytest.raises(moon.context.HipError):
+            dev.greedy(2)
+        dev.reset()
+        dev.forward(ids)
+        assert dev.greedy(6).tolist() == want, f"decode mode {mode} after a reset"
+    dev.close()
+
+
+def test_streaming_decode_kernel_against_the_per_layer_kernels(moon, O, ctx):
+    """Decode mode 4 (one launch for the whole greedy loop, weights streamed through LDS rings, workgroups exchanging q/k/v,
+    attention partials, partial sums and the hidden state through tagged words): same ids as the per-layer kernels, hidden
+    state and logits within the end-to-end bound of theirs (out_proj and fc2 are summed in another order), single steps,
+    a run up to the last cache position, and interleaving with forward() calls."""
+    dev = moon.text_model.TextModel(moon.text_model.default_config(), seed=0, std=0.02, ctx=ctx)
+    ids = O.fill_uniform_u32(50, 0, 50, 51200)
     dev.forward(ids)
-    ctx.check(ctx.lib.moon_text_debug_raise_wait_error(dev.handle))
-    with pytest.raises(moon.context.HipError):
-        dev.greedy(2)
+    want = dev.greedy(20).tolist()
+    want_hidden, want_logits = dev.hidden(1).copy(), dev.logits().copy()
     dev.reset()
+    dev.set_decode_mode(4)
     dev.forward(ids)
-    assert dev.greedy(6).tolist() == want
+    got = dev.greedy(1).tolist() + dev.greedy(1).tolist() + dev.greedy(18).tolist()
+    assert got == want
+    assert dev.position == 70
+    assert O.rel_frobenius(dev.hidden(1), want_hidden) <= 4 * TOL
+    assert O.rel_frobenius(dev.logits().reshape(1, -1), want_logits.reshape(1, -1)) <= 4 * TOL
+    # a prompt continuation through forward(), then the loop again: both paths read and extend the same cache
+    more = O.fill_uniform_u32(7, 0, 51, 51200)
+    dev.forward(more)
+    a = dev.greedy(5).tolist()
+    dev.reset()
+    dev.set_decode_mode(0)
+    dev.forward(ids)
+    dev.greedy(20)
+    dev.forward(more)
+    assert dev.greedy(5).tolist() == a
+    # up to the last position of the cache (2048), and not beyond
+    dev.reset()
+    dev.set_decode_mode(4)
+    dev.forward(O.fill_uniform_u32(2040, 0, 52, 51200))
+    b4 = dev.greedy(8).tolist()
+    assert dev.position == 2048
+    with pytest.raises(moon.SequenceTooLong):
+        dev.greedy(1)
+    dev.reset()
+    dev.set_decode_mode(0)
+    dev.forward(O.fill_uniform_u32(2040, 0, 52, 51200))
+    assert dev.greedy(8).tolist() == b4
     dev.close()
