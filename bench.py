@@ -380,6 +380,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-extra", action="store_true", help="skip the GEMM / attention / vision side measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-gemm", action="store_true",
+                    help="only the stand-alone GEMM / attention / vision legs, printed as their own JSON line (what a counter run profiles)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run 8 plain 256 MiB copies (copy16_kernel) as the known-traffic yardstick for a counter run")
     ap.add_argument("--decode-mode", type=int, default=None,
@@ -394,6 +396,14 @@ def main():
     ctx = moon.Context(0)
     if args.calibrate_copy:
         calibration_copies(ctx)
+    if args.only_gemm:
+        out = {"gemm_vision_fc1": bench_gemm(moon, ctx, 729, 1152, 4304), "gemm_vision_fc2": bench_gemm(moon, ctx, 729, 4304, 1152),
+               "gemm_vision_qkv": bench_gemm(moon, ctx, 729, 1152, 3456), "gemm_vision_fc1_m1458": bench_gemm(moon, ctx, 1458, 1152, 4304),
+               "gemm_prefill_fc1": bench_gemm(moon, ctx, 768, 2048, 8192), "attention": bench_attention(moon, ctx),
+               "vision_encoder_27_blocks": bench_vision(moon, ctx)}
+        ctx.close()
+        print(json.dumps(out))
+        return
     model, dec = bench_decoder(moon, ctx, args.steps, args.warmup, args.decode_mode)
     kern = profile_decode_kernels(model, dec["ms_per_token"] * 1e3, args.decode_mode)
     sampled = None if args.no_extra else bench_sampled_decode(moon, ctx, model)

@@ -748,6 +748,80 @@ __global__ __launch_bounds__(256) void splitk_reduce8_kernel(const float *__rest
     *reinterpret_cast<half8_t *>(C + i) = o;
 }
 
+// The split-K reduction followed by the LayerNorm of the finished rows, one wavefront per row of C (N <= 2048, N % 8 == 0):
+// the sums and the epilogue are those of splitk_reduce8_kernel (same order over the splits); the row stays in registers
+// and ops.layerNorm (ops.zig:1063-1419: f32 mean, biased variance, y = f16((x*rstd - mean*rstd)*gamma + beta)) is applied
+// to the f16 values just written to C, into ln_out.  Replaces a LayerNorm launch that would re-read C.
+constexpr int LN_FUSE_MAX_N = 2048;
+template <int EPI>
+__global__ __launch_bounds__(256) void splitk_reduce_ln_kernel(const float *__restrict__ partial, const half_t *__restrict__ bias, const half_t *resid,
+                                                               half_t *C, const half_t *__restrict__ gamma, const half_t *__restrict__ beta,
+                                                               half_t *__restrict__ ln_out, int M, int N, int splits, float eps) {
+    const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const size_t MN = size_t(M) * N, base = size_t(row) * N;
+    half8_t v[LN_FUSE_MAX_N / 512];
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < LN_FUSE_MAX_N / 512; j++) {
+        const int n = lane * 8 + 512 * j;
+        v[j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        if (n < N) {
+            const size_t i = base + n;
+            float4 a = *reinterpret_cast<const float4 *>(partial + i), b = *reinterpret_cast<const float4 *>(partial + i + 4);
+            for (int k = 1; k < splits; k++) {
+                const float4 c = *reinterpret_cast<const float4 *>(partial + size_t(k) * MN + i),
+                             d = *reinterpret_cast<const float4 *>(partial + size_t(k) * MN + i + 4);
+                a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
+                b.x += d.x; b.y += d.y; b.z += d.z; b.w += d.w;
+            }
+            const float s[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+            half8_t bv = {0, 0, 0, 0, 0, 0, 0, 0}, rv = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (EPI >= MOON_EPI_BIAS) bv = *reinterpret_cast<const half8_t *>(bias + n);
+            if (EPI == MOON_EPI_BIAS_RESID) rv = *reinterpret_cast<const half8_t *>(resid + i);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                half_t o = apply_epilogue_v<EPI>(s[e], bv[e]);
+                if (EPI == MOON_EPI_BIAS_RESID) o = (half_t)((float)rv[e] + (float)o);
+                v[j][e] = o;
+                sum += (float)o;
+            }
+            *reinterpret_cast<half8_t *>(C + i) = v[j];
+        }
+    }
+    const float mean = wave_sum(sum) / (float)N;
+    float m2 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < LN_FUSE_MAX_N / 512; j++)
+        if (lane * 8 + 512 * j < N) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float d = (float)v[j][e] - mean;
+                m2 = fmaf(d, d, m2);
+            }
+        }
+    const float var = wave_sum(m2) / (float)N;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    {
+#pragma clang fp contract(off)
+        const float mean_rstd = mean * rstd; // ops.zig:1301, 1330-1333: separate multiplies and adds
+#pragma unroll
+        for (int j = 0; j < LN_FUSE_MAX_N / 512; j++) {
+            const int n = lane * 8 + 512 * j;
+            if (n < N) {
+                const half8_t g = *reinterpret_cast<const half8_t *>(gamma + n), bt = *reinterpret_cast<const half8_t *>(beta + n);
+                half8_t o;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float x = (float)v[j][e] * rstd - mean_rstd;
+                    o[e] = (half_t)(x * (float)g[e] + (float)bt[e]);
+                }
+                *reinterpret_cast<half8_t *>(ln_out + base + n) = o;
+            }
+        }
+    }
+}
+
 // Any shape / alignment: one thread per output, sequential-k f32 accumulation.
 template <int EPI>
 __global__ void gemm_generic_kernel(const half_t *__restrict__ A, const half_t *__restrict__ B, const half_t *__restrict__ bias,
@@ -778,9 +852,11 @@ __global__ __launch_bounds__(256) void transpose_kernel(const half_t *__restrict
     }
 }
 
+// ln: optional LayerNorm of the finished rows of C into ln->out.  *ln_done says whether it was fused (into the split-K
+// reduction); if not, the caller runs it as a launch of its own.
 template <int EPI>
 int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias, const half_t *resid, half_t *C, int M, int N, int K,
-             int b_layout) {
+             int b_layout, const GemmLayerNorm *ln, bool *ln_done) {
     const bool aligned = (K % 8 == 0) && (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 8 == 0) && K > 0;
     if (!aligned) {
@@ -887,7 +963,13 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     MOON_HIP(ctx, hipGetLastError());
     if (splits > 1) {
         const size_t mn = size_t(M) * N;
-        if (N % 8 == 0 && p.lds_epilogue)
+        const bool ln_ok = ln && N % 8 == 0 && N <= LN_FUSE_MAX_N && p.lds_epilogue && reinterpret_cast<uintptr_t>(ln->gamma) % 16 == 0 &&
+                           reinterpret_cast<uintptr_t>(ln->beta) % 16 == 0 && reinterpret_cast<uintptr_t>(ln->out) % 16 == 0;
+        if (ln_ok) {
+            hipLaunchKernelGGL(splitk_reduce_ln_kernel<EPI>, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, ctx->stream, p.partial, bias, resid, C,
+                               ln->gamma, ln->beta, ln->out, M, N, splits, ln->eps);
+            *ln_done = true;
+        } else if (N % 8 == 0 && p.lds_epilogue)
             hipLaunchKernelGGL(splitk_reduce8_kernel<EPI>, dim3((unsigned)((mn / 8 + 255) / 256)), dim3(256), 0, ctx->stream, p.partial, bias,
                                resid, C, mn, N, splits);
         else
@@ -901,20 +983,27 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
 } // namespace
 
 int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias, half_t *C, size_t M, size_t N, size_t K,
-                int b_layout, int epilogue, const half_t *resid) {
+                int b_layout, int epilogue, const half_t *resid, const GemmLayerNorm *ln) {
     if (M == 0 || N == 0) return MOON_OK;
     if (M > 0x3fffffff || N > 0x3fffffff || K > 0x3fffffff) return moon_fail(ctx, MOON_EINVAL_DIM, "gemm: dimension too large");
     if (epilogue != MOON_EPI_NONE && !bias) return moon_fail(ctx, MOON_EINVAL, "gemm: epilogue needs a bias");
     if (b_layout != MOON_B_KN && b_layout != MOON_B_NK) return moon_fail(ctx, MOON_EINVAL, "gemm: unknown B layout %d", b_layout);
+    if (ln && (!ln->gamma || !ln->beta || !ln->out)) return moon_fail(ctx, MOON_EINVAL, "gemm: the LayerNorm that follows needs gamma, beta and an output");
+    if (ln && !(ln->eps > 0.0f)) return moon_fail(ctx, MOON_EEPS, "gemm: the LayerNorm that follows needs eps > 0");
+    bool ln_done = false;
+    int rc;
     switch (epilogue) {
-    case MOON_EPI_NONE: return run_gemm<MOON_EPI_NONE>(ctx, A, B, bias, nullptr, C, (int)M, (int)N, (int)K, b_layout);
-    case MOON_EPI_BIAS: return run_gemm<MOON_EPI_BIAS>(ctx, A, B, bias, nullptr, C, (int)M, (int)N, (int)K, b_layout);
-    case MOON_EPI_BIAS_GELU: return run_gemm<MOON_EPI_BIAS_GELU>(ctx, A, B, bias, nullptr, C, (int)M, (int)N, (int)K, b_layout);
+    case MOON_EPI_NONE: rc = run_gemm<MOON_EPI_NONE>(ctx, A, B, bias, nullptr, C, (int)M, (int)N, (int)K, b_layout, ln, &ln_done); break;
+    case MOON_EPI_BIAS: rc = run_gemm<MOON_EPI_BIAS>(ctx, A, B, bias, nullptr, C, (int)M, (int)N, (int)K, b_layout, ln, &ln_done); break;
+    case MOON_EPI_BIAS_GELU: rc = run_gemm<MOON_EPI_BIAS_GELU>(ctx, A, B, bias, nullptr, C, (int)M, (int)N, (int)K, b_layout, ln, &ln_done); break;
     case MOON_EPI_BIAS_RESID:
         if (!resid) return moon_fail(ctx, MOON_EINVAL, "gemm: the residual epilogue needs a residual");
-        return run_gemm<MOON_EPI_BIAS_RESID>(ctx, A, B, bias, resid, C, (int)M, (int)N, (int)K, b_layout);
+        rc = run_gemm<MOON_EPI_BIAS_RESID>(ctx, A, B, bias, resid, C, (int)M, (int)N, (int)K, b_layout, ln, &ln_done);
+        break;
     default: return moon_fail(ctx, MOON_EINVAL, "gemm: unknown epilogue %d", epilogue);
     }
+    if (rc != MOON_OK || !ln || ln_done) return rc;
+    return launch_layernorm(ctx, C, ln->gamma, ln->beta, ln->out, M, N, ln->eps);
 }
 
 // dst[cols, rows] = src[rows, cols]^T

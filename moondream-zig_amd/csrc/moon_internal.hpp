@@ -67,8 +67,15 @@ int launch_gemv_nt(moon_ctx *ctx, const half_t *x, const half_t *W, const half_t
                    size_t N, size_t K, int epilogue);
 // C[M,N] = epi(A[M,K] x B) with B[N,K] (b_layout NK) or B[K,N] (KN); MFMA kernel, generic fallback for odd K.
 // epilogue: a MOON_EPI_* value, or the internal MOON_EPI_BIAS_RESID (3): C = f16(resid + f16(f16(acc) + bias)), resid may be C.
+// ln: a LayerNorm of the finished rows of C into ln->out (the reference's next op on this tensor, vision_model.zig:239, 253,
+// 266): fused into the split-K reduction where the product takes that path, a launch of its own otherwise.
+struct GemmLayerNorm {
+    const half_t *gamma, *beta;
+    half_t *out;
+    float eps;
+};
 int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias, half_t *C,
-                size_t M, size_t N, size_t K, int b_layout, int epilogue, const half_t *resid = nullptr);
+                size_t M, size_t N, size_t K, int b_layout, int epilogue, const half_t *resid = nullptr, const GemmLayerNorm *ln = nullptr);
 
 int launch_layernorm(moon_ctx *ctx, const half_t *x, const half_t *gamma, const half_t *beta, half_t *y,
                      size_t rows, size_t dim, float eps);

@@ -104,9 +104,13 @@ int encode_dev(moon_vision_model *m, const half_t *x_in, size_t T, half_t *out) 
     const size_t d = m->cfg.dim, f = m->cfg.hidden_dim, H = m->cfg.n_heads, D = m->cfg.head_dim;
     MOON_TRY(ensure_activations(m, T));
     MOON_HIP(ctx, hipMemcpyAsync(m->x, x_in, T * d * sizeof(half_t), hipMemcpyDeviceToDevice, ctx->stream));
+    // Every LayerNorm but the first follows a product that has just finished the rows it normalises (out_proj + residual ->
+    // ln2; fc2 + residual -> the next block's ln1, or the final LayerNorm): it is handed to that product, which folds it into
+    // its split-K reduction where it has one (launch_gemm), instead of a launch that re-reads x.
+    if (m->cfg.n_layers == 0) return launch_layernorm(ctx, m->x, m->no_w, m->no_b, out, T, d, m->cfg.ln_eps);
+    MOON_TRY(launch_layernorm(ctx, m->x, m->n1_w, m->n1_b, m->ln, T, d, m->cfg.ln_eps));
     for (size_t l = 0; l < m->cfg.n_layers; l++) {
         // x += attention_block(layerNorm(x))   (vision_model.zig:239-248)
-        MOON_TRY(launch_layernorm(ctx, m->x, m->n1_w + l * d, m->n1_b + l * d, m->ln, T, d, m->cfg.ln_eps));
         MOON_TRY(launch_gemm(ctx, m->ln, m->qkv_w + l * 3 * d * d, m->qkv_b + l * 3 * d, m->qkv, T, 3 * d, d, MOON_B_NK, MOON_EPI_BIAS));
         bool packed = false; // the matrix-core kernel reads q, k, v in place; other shapes are split into [H, T, D] tensors first
         MOON_TRY(launch_sdpa_packed_qkv(ctx, m->qkv, m->attn, H, T, D, &packed));
@@ -116,13 +120,15 @@ int encode_dev(moon_vision_model *m, const half_t *x_in, size_t T, half_t *out) 
             MOON_TRY(launch_split_heads(ctx, m->qkv, 3 * d, 2 * d, m->v, T, H, D));
             MOON_TRY(launch_sdpa(ctx, m->q, m->k, m->v, m->attn, H, T, T, D, T * D, -1, nullptr, 0, true));
         }
-        MOON_TRY(launch_gemm(ctx, m->attn, m->out_w + l * d * d, m->out_b + l * d, m->x, T, d, d, MOON_B_NK, 3 /* bias, then += into x */, m->x));
         // x += mlp(layerNorm(x))               (vision_model.zig:253-262)
-        MOON_TRY(launch_layernorm(ctx, m->x, m->n2_w + l * d, m->n2_b + l * d, m->ln, T, d, m->cfg.ln_eps));
+        const GemmLayerNorm ln2{m->n2_w + l * d, m->n2_b + l * d, m->ln, m->cfg.ln_eps};
+        MOON_TRY(launch_gemm(ctx, m->attn, m->out_w + l * d * d, m->out_b + l * d, m->x, T, d, d, MOON_B_NK, 3 /* bias, then += into x */, m->x, &ln2));
         MOON_TRY(launch_gemm(ctx, m->ln, m->fc1_w + l * d * f, m->fc1_b + l * f, m->fc1, T, f, d, MOON_B_NK, MOON_EPI_BIAS_GELU));
-        MOON_TRY(launch_gemm(ctx, m->fc1, m->fc2_w + l * f * d, m->fc2_b + l * d, m->x, T, d, f, MOON_B_NK, 3 /* bias, then += into x */, m->x));
+        const bool last = l + 1 == m->cfg.n_layers; // the final LayerNorm (vision_model.zig:266) or the next block's first
+        const GemmLayerNorm next{last ? m->no_w : m->n1_w + (l + 1) * d, last ? m->no_b : m->n1_b + (l + 1) * d, last ? out : m->ln, m->cfg.ln_eps};
+        MOON_TRY(launch_gemm(ctx, m->fc1, m->fc2_w + l * f * d, m->fc2_b + l * d, m->x, T, d, f, MOON_B_NK, 3 /* bias, then += into x */, m->x, &next));
     }
-    return launch_layernorm(ctx, m->x, m->no_w, m->no_b, out, T, d, m->cfg.ln_eps); // vision_model.zig:266
+    return MOON_OK;
 }
 
 // encode_image (vision_model.zig:186-229): patches[2T, patch_dim] on the device -> out[T, out_dim] on the device
