@@ -161,11 +161,18 @@ int moon_image_patches(moon_ctx *ctx, const uint8_t *image, size_t height, size_
 void moon_sampling_config_default(moon_sampling_config *cfg);
 /* sampling.sample(&f32(logits), config, rng, allocator) (sampling.zig:353-389, called at moondream.zig:335-337 and
  * moonchat.zig:597) on one row of n logits.  The reference draws one number per call from its PRNG,
- * rng.float(f32) in [0,1): pass it as u (unused by greedy); the generator stays with the caller.  Sums over the whole
- * vocabulary are taken in another order than the reference's sequential loops, which can move the boundary between
- * two neighbouring candidates by about 1e-7 of the total; apart from a u that close to a boundary the index is the
- * reference's. */
+ * rng.float(f32) in [0,1): pass it as u (unused by greedy); the generator stays with the caller.  The reference's sums
+ * over the vocabulary are sequential f32 loops, and the candidate a draw lands on depends on their rounding: the device
+ * evaluates those loops bit for bit, so for the same exps the index is the reference's for every u.  (exp itself is the
+ * classic two-part-reduction expf, error below one ulp, spelled out in csrc/sample.hip; a libm whose expf rounds some
+ * argument differently can move a boundary by that last bit.)  top_k sorts at most 1024 candidates on the device: a
+ * larger min(top_k, n) is refused with MOON_EINVAL, a deliberate limit (the reference's CLI default is 3). */
 int moon_sample(moon_ctx *ctx, const moon_f16 *logits, size_t n, const moon_sampling_config *cfg, float u, size_t *index);
+/* The same on the f32 row the reference's signature takes (sample(tensor: *Tensor(f32), ...), sampling.zig:353-358; at its
+ * call sites the row is the f16 LM-head output cast to f32, moondream.zig:335): any f32 values are accepted. */
+int moon_sample_f32(moon_ctx *ctx, const float *logits, size_t n, const moon_sampling_config *cfg, float u, size_t *index);
+/* sampling.argmax(f32, tensor) (sampling.zig:257-273): first maximum wins. */
+int moon_argmax_f32(moon_ctx *ctx, const float *logits, size_t n, size_t *index);
 
 /* ------------------------------------------------------------------ device memory + device-pointer ops
  * The same kernels, on buffers that already live in HBM (what the benchmark times and what the
@@ -366,7 +373,10 @@ typedef struct moon_bin moon_bin;
 int moon_bin_open(const char *path, moon_bin **out, char *err, size_t err_len);
 void moon_bin_close(moon_bin *bin);
 size_t moon_bin_tensor_count(const moon_bin *bin);
-/* tensor by position in the file / by name (MOON_EFORMAT if absent); any output pointer may be NULL */
+/* tensor by position in the file / by name (MOON_EFORMAT if absent); any output pointer may be NULL.  A record's element
+ * count must agree with its dimensions and fit the file (MOON_EFORMAT otherwise).  The data pointer addresses the bytes
+ * where they lie in the file, after a name of any length: it may be odd, so copy from it (memcpy, moon_dev_upload, the
+ * weight structs' consumers do) rather than dereference it as moon_f16. */
 int moon_bin_tensor(const moon_bin *bin, size_t index, const char **name, size_t *ndim, size_t dims[4], const moon_f16 **data);
 int moon_bin_find(const moon_bin *bin, const char *name, size_t *ndim, size_t dims[4], const moon_f16 **data);
 /* Fill the weight structs of the sessions above from the file, checking every shape against the configuration exactly as
@@ -376,6 +386,20 @@ int moon_bin_text_weights(const moon_bin *bin, const moon_text_config *cfg, moon
 int moon_bin_vision_weights(const moon_bin *bin, const moon_vision_config *cfg, moon_vision_weights *w, char *err, size_t err_len);
 int moon_bin_vision_io_weights(const moon_bin *bin, const moon_vision_config *cfg, const moon_vision_io_config *io,
                                moon_vision_io_weights *w, char *err, size_t err_len);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Environment variables.  None is needed: the defaults are what the tests and the bench run.  They are tuning and
+ * diagnostic aids, read once per process (the first call that looks at them fixes the value for every context):
+ *   MOON_DECODE_TRACE=1            text sessions record per-workgroup time stamps of the last layer launch of a greedy call
+ *                                  and print a per-role timeline to stderr (allocated at session creation)
+ *   MOON_STREAM_DEBUG=n            decode mode 4 only: switches parts of the streaming kernel off (timing experiments; wrong results)
+ *   MOON_LAYER_OUT_CHUNK=1|2|4|8|16  decode mode 0: 1 KiB pieces of an fc2 row an output wavefront requests before it waits (default 4)
+ *   MOON_LAYER_QKV_WGS=n           decode mode 0: workgroups that take qkv rows (default: the attention and output workgroups)
+ *   MOON_LAYER_FC1_OUT_ROWS=n      decode mode 0: fc1 rows per output wavefront (default: half an fc1-only wavefront's share)
+ *   MOON_LAYER_FC1_GROUP=1|2       decode mode 0: fc1 rows a wavefront requests together (default 1)
+ *   MOON_GEMM_KERNEL=regs|dma|dma256  forces one of the MFMA product kernels where the shape allows it (default: by shape)
+ *   MOON_GEMM_EPILOGUE=direct      the product kernels store their tile without the pass through LDS (default: through LDS)
+ * Every setting gives the same results (bit for bit, MOON_STREAM_DEBUG aside); only the time changes. */
 
 #ifdef __cplusplus
 }

@@ -89,6 +89,8 @@ SIGNATURES = {
     "moon_image_patches": (_i, [_vp, _vp, _sz, _sz, _sz, _sz, _vp]),
     "moon_sampling_config_default": (None, [_vp]),
     "moon_sample": (_i, [_vp, _vp, _sz, _vp, _f, C.POINTER(_sz)]),
+    "moon_sample_f32": (_i, [_vp, _vp, _sz, _vp, _f, C.POINTER(_sz)]),
+    "moon_argmax_f32": (_i, [_vp, _vp, _sz, C.POINTER(_sz)]),
     "moon_dev_sample": (_i, [_vp, _vp, _sz, _vp, _f, C.POINTER(_sz)]),
     "moon_dev_alloc": (_i, [_vp, _sz, _pp]),
     "moon_dev_free": (_i, [_vp, _vp]),

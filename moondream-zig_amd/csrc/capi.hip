@@ -29,11 +29,31 @@ int fetch(moon_ctx *ctx, void *host, const void *dptr, size_t bytes) {
     return MOON_OK;
 }
 
-// resident weight if this exact host buffer was registered, else a staged copy
-int weight_in(moon_ctx *ctx, int slot, const moon_f16 *host, size_t n_elems, const half_t **dptr) {
+// resident weight if this exact host buffer was registered, else a staged copy.  A registered weight that is used as
+// B[K,N] (hgemm.matmul's layout, hgemm.zig:210-216) gets an [N,K] copy on its first such use, kept until it is
+// unregistered, and *b_layout becomes MOON_B_NK: the product then runs without a transpose pass per call.
+int weight_in(moon_ctx *ctx, int slot, const moon_f16 *host, size_t n_elems, const half_t **dptr, int *b_layout = nullptr, size_t K = 0,
+              size_t N = 0) {
     auto it = ctx->resident.find(host);
     if (it != ctx->resident.end() && it->second.n_elems == n_elems) {
-        *dptr = (const half_t *)it->second.dptr;
+        moon_ctx::Resident &r = it->second;
+        if (b_layout && *b_layout == MOON_B_KN && K * N == n_elems && K > 1 && N > 1) {
+            if (!r.dptr_t || r.t_k != K || r.t_n != N) {
+                if (r.dptr_t) {
+                    MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
+                    MOON_HIP(ctx, hipFree(r.dptr_t));
+                    r.dptr_t = nullptr;
+                }
+                MOON_HIP(ctx, hipMalloc(&r.dptr_t, n_elems * sizeof(moon_f16)));
+                MOON_TRY(launch_transpose(ctx, (const half_t *)r.dptr, (half_t *)r.dptr_t, K, N));
+                r.t_k = K;
+                r.t_n = N;
+            }
+            *dptr = (const half_t *)r.dptr_t;
+            *b_layout = MOON_B_NK;
+            return MOON_OK;
+        }
+        *dptr = (const half_t *)r.dptr;
         return MOON_OK;
     }
     void *d = nullptr;
@@ -59,7 +79,7 @@ int linear_host(moon_ctx *ctx, const moon_f16 *a, size_t M, size_t K, const moon
     void *da = nullptr, *dc = nullptr, *dbias = nullptr;
     const half_t *db = nullptr;
     MOON_TRY(stage_in(ctx, ST_A, a, M * K * sizeof(moon_f16), &da));
-    MOON_TRY(weight_in(ctx, ST_B, b, N * K, &db));
+    MOON_TRY(weight_in(ctx, ST_B, b, N * K, &db, &b_layout, K, N));
     if (bias) MOON_TRY(stage_in(ctx, ST_AUX, bias, N * sizeof(moon_f16), &dbias));
     MOON_TRY(stage_out(ctx, ST_C, M * N * sizeof(moon_f16), &dc));
     MOON_TRY(linear_dev(ctx, (const half_t *)da, M, K, db, N, b_layout, (const half_t *)dbias, epilogue, (half_t *)dc));
@@ -326,6 +346,41 @@ extern "C" int moon_dev_sample(moon_ctx *ctx, const void *logits, size_t n, cons
     if (!n) return moon_fail(ctx, MOON_EINVAL, "dev_sample: empty tensor (EmptyTensor)");
     MOON_HIP(ctx, hipSetDevice(ctx->device));
     return sample_dev(ctx, (const half_t *)logits, n, cfg, u, index);
+}
+
+extern "C" int moon_sample_f32(moon_ctx *ctx, const float *logits, size_t n, const moon_sampling_config *cfg, float u, size_t *index) {
+    if (!ctx) return MOON_EINVAL;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (!logits || !index || !cfg) return moon_fail(ctx, MOON_EINVAL, "sample_f32: null operand");
+    if (!n) return moon_fail(ctx, MOON_EINVAL, "sample_f32: empty tensor (EmptyTensor)");
+    MOON_HIP(ctx, hipSetDevice(ctx->device));
+    void *dl, *di;
+    MOON_TRY(stage_in(ctx, ST_A, logits, n * sizeof(float), &dl));
+    MOON_TRY(stage_out(ctx, ST_C, sizeof(uint32_t), &di));
+    if (cfg->method == MOON_SAMPLE_GREEDY)
+        MOON_TRY(launch_argmax_f32(ctx, (const float *)dl, n, (uint32_t *)di));
+    else
+        MOON_TRY(launch_sample(ctx, nullptr, n, cfg, u, nullptr, nullptr, nullptr, (uint32_t *)di, 0, (const float *)dl));
+    uint32_t idx = 0;
+    MOON_TRY(fetch(ctx, &idx, di, sizeof(idx)));
+    *index = idx;
+    return MOON_OK;
+}
+
+extern "C" int moon_argmax_f32(moon_ctx *ctx, const float *logits, size_t n, size_t *index) {
+    if (!ctx) return MOON_EINVAL;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (!logits || !index) return moon_fail(ctx, MOON_EINVAL, "argmax_f32: null operand");
+    if (!n) return moon_fail(ctx, MOON_EINVAL, "argmax_f32: empty tensor (EmptyTensor)");
+    MOON_HIP(ctx, hipSetDevice(ctx->device));
+    void *dl, *di;
+    MOON_TRY(stage_in(ctx, ST_A, logits, n * sizeof(float), &dl));
+    MOON_TRY(stage_out(ctx, ST_C, sizeof(uint32_t), &di));
+    MOON_TRY(launch_argmax_f32(ctx, (const float *)dl, n, (uint32_t *)di));
+    uint32_t idx = 0;
+    MOON_TRY(fetch(ctx, &idx, di, sizeof(idx)));
+    *index = idx;
+    return MOON_OK;
 }
 
 // ------------------------------------------------------------------ device-pointer ops

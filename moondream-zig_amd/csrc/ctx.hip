@@ -84,7 +84,10 @@ extern "C" void moon_cleanup(moon_ctx *ctx) {
 extern "C" void moon_ctx_destroy(moon_ctx *ctx) {
     if (!ctx) return;
     moon_cleanup(ctx);
-    for (auto &kv : ctx->resident) (void)hipFree(kv.second.dptr);
+    for (auto &kv : ctx->resident) {
+        (void)hipFree(kv.second.dptr);
+        if (kv.second.dptr_t) (void)hipFree(kv.second.dptr_t);
+    }
     ctx->resident.clear();
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
@@ -146,6 +149,7 @@ extern "C" int moon_weight_register(moon_ctx *ctx, const moon_f16 *host, size_t 
     if (it != ctx->resident.end()) {
         MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
         MOON_HIP(ctx, hipFree(it->second.dptr));
+        if (it->second.dptr_t) MOON_HIP(ctx, hipFree(it->second.dptr_t));
         ctx->resident.erase(it);
     }
     void *d = nullptr;
@@ -156,7 +160,7 @@ extern "C" int moon_weight_register(moon_ctx *ctx, const moon_f16 *host, size_t 
         (void)hipFree(d);
         return moon_fail(ctx, MOON_EHIP, "weight upload: %s", hipGetErrorString(e));
     }
-    ctx->resident[host] = {d, n_elems};
+    ctx->resident[host] = moon_ctx::Resident{d, n_elems};
     return MOON_OK;
 }
 
@@ -167,6 +171,7 @@ extern "C" int moon_weight_unregister(moon_ctx *ctx, const moon_f16 *host) {
     if (it == ctx->resident.end()) return moon_fail(ctx, MOON_EINVAL, "moon_weight_unregister: pointer was not registered");
     MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
     MOON_HIP(ctx, hipFree(it->second.dptr));
+    if (it->second.dptr_t) MOON_HIP(ctx, hipFree(it->second.dptr_t));
     ctx->resident.erase(it);
     return MOON_OK;
 }

@@ -42,7 +42,8 @@ __global__ void residual2_kernel(half_t *hidden, const half_t *__restrict__ attn
 
 // sampling.argmax (sampling.zig:257-273): strict '>' scan from index 0, i.e. the lowest index among
 // equal maxima; NaN never wins.  Single workgroup (51200 logits = 100 KiB).
-__global__ __launch_bounds__(1024) void argmax_kernel(const half_t *__restrict__ logits, int n, uint32_t *out) {
+template <class T>
+__global__ __launch_bounds__(1024) void argmax_kernel(const T *__restrict__ logits, int n, uint32_t *out) {
     __shared__ float sv[16];
     __shared__ int si[16];
     float best = -INFINITY;
@@ -264,7 +265,13 @@ int launch_image_patches(moon_ctx *ctx, const uint8_t *image, half_t *out, size_
 
 int launch_argmax(moon_ctx *ctx, const half_t *logits, size_t n, uint32_t *index_out) {
     if (!n || n > 0x7fffffff) return moon_fail(ctx, MOON_EINVAL, "argmax: empty or oversized tensor");
-    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, ctx->stream, logits, (int)n, index_out);
+    hipLaunchKernelGGL(argmax_kernel<half_t>, dim3(1), dim3(1024), 0, ctx->stream, logits, (int)n, index_out);
+    MOON_HIP(ctx, hipGetLastError());
+    return MOON_OK;
+}
+int launch_argmax_f32(moon_ctx *ctx, const float *logits, size_t n, uint32_t *index_out) {
+    if (!n || n > 0x7fffffff) return moon_fail(ctx, MOON_EINVAL, "argmax: empty or oversized tensor");
+    hipLaunchKernelGGL(argmax_kernel<float>, dim3(1), dim3(1024), 0, ctx->stream, logits, (int)n, index_out);
     MOON_HIP(ctx, hipGetLastError());
     return MOON_OK;
 }

@@ -16,6 +16,7 @@
 // workspace; resident model weights are transposed once at load time instead.
 // Small grids (tiles < CUs) split K across workgroups: f32 partials to a workspace, then a fixed-order
 // reduction applies the epilogue (deterministic, no atomics).
+#include <atomic>
 #include <cstring>
 
 #include "epilogue.hpp"
@@ -911,11 +912,13 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
         p.k_per_split = K;
         const int total = p.tiles_m * p.tiles_n;
         const size_t lds_bytes = use192 ? Dma2<3>::LDS_BYTES : Dma2<4>::LDS_BYTES;
-        static bool attr_set[2] = {false, false}; // (per instantiation of this function, i.e. per epilogue)
-        if (!attr_set[use192 ? 1 : 0]) {
+        // the opt-in to this much dynamic LDS is per device and per kernel (here: per epilogue instantiation); setting it twice is harmless
+        static std::atomic<bool> attr_set[2][64];
+        const int dev = ctx->device >= 0 && ctx->device < 64 ? ctx->device : -1;
+        if (dev < 0 || !attr_set[use192 ? 1 : 0][dev].load()) {
             const void *kern = use192 ? reinterpret_cast<const void *>(gemm_nt_dma192_kernel<EPI>) : reinterpret_cast<const void *>(gemm_nt_dma256_kernel<EPI>);
             MOON_HIP(ctx, hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-            attr_set[use192 ? 1 : 0] = true;
+            if (dev >= 0) attr_set[use192 ? 1 : 0][dev].store(true);
         }
         const dim3 grid2(((total + 7) / 8) * 8);
         if (use192) hipLaunchKernelGGL(gemm_nt_dma192_kernel<EPI>, grid2, dim3(DMA_THREADS), lds_bytes, ctx->stream, p);
@@ -950,11 +953,12 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     if (force && !strcmp(force, "regs")) use_dma = false;
     if (force && !strcmp(force, "dma")) use_dma = K % 16 == 0 && buffers_ok;
     if (use_dma) {
-        static bool attr_set = false; // 128 KiB of dynamic LDS needs the opt-in once per process (per instantiation)
-        if (!attr_set) {
+        static std::atomic<bool> attr_set[64]; // 128 KiB of dynamic LDS needs the opt-in once per device (and per instantiation)
+        const int dev = ctx->device >= 0 && ctx->device < 64 ? ctx->device : -1;
+        if (dev < 0 || !attr_set[dev].load()) {
             MOON_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_nt_dma_kernel<EPI>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)DMA_LDS_BYTES));
-            attr_set = true;
+            if (dev >= 0) attr_set[dev].store(true);
         }
         hipLaunchKernelGGL(gemm_nt_dma_kernel<EPI>, dim3(grid), dim3(DMA_THREADS), DMA_LDS_BYTES, ctx->stream, p);
     } else {

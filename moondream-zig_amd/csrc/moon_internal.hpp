@@ -39,6 +39,8 @@ struct moon_ctx {
     struct Resident {
         void *dptr;
         size_t n_elems;
+        void *dptr_t = nullptr;    // [N,K] copy of a weight used as B[K,N] (hgemm.matmul's layout), made on its first such use
+        size_t t_k = 0, t_n = 0;
     };
     std::map<const void *, Resident> resident;
 };
@@ -85,12 +87,14 @@ int launch_add(moon_ctx *ctx, half_t *a, const half_t *b, size_t n);
 // a = f16(a + f16(b + c))  -- the parallel-block residual (text_model.zig:170-171)
 int launch_residual2(moon_ctx *ctx, half_t *hidden, const half_t *attn, const half_t *mlp, size_t n);
 int launch_argmax(moon_ctx *ctx, const half_t *logits, size_t n, uint32_t *index_out);
+int launch_argmax_f32(moon_ctx *ctx, const float *logits, size_t n, uint32_t *index_out);
 // resized u8 image [H,W,C] -> normalised f16 patches [copies * (H/P)*(W/P), C*P*P], rows `pitch` halfs apart
 int launch_image_patches(moon_ctx *ctx, const uint8_t *image, half_t *out, size_t H, size_t W, size_t C, size_t P, size_t copies, size_t pitch);
+// logits_f32: the row as f32 instead of f16 (then logits is unused).
 // sampling.sample for the methods other than greedy: u, or u_dev[state ? state[1] : 0] when u_dev is set; the token goes to
 // out[0] (if out) and, if state, to state[2] and out_ids[state[1]++], and state[0] += bump_pos (the decode loop's bookkeeping).
 int launch_sample(moon_ctx *ctx, const half_t *logits, size_t n, const moon_sampling_config *cfg, float u, const float *u_dev,
-                  uint32_t *state, uint32_t *out_ids, uint32_t *out, uint32_t bump_pos = 0);
+                  uint32_t *state, uint32_t *out_ids, uint32_t *out, uint32_t bump_pos = 0, const float *logits_f32 = nullptr);
 int launch_embed(moon_ctx *ctx, const half_t *wte, const uint32_t *ids, half_t *out, size_t n_ids, size_t dim);
 int launch_rope_table(moon_ctx *ctx, float *table, size_t rot_dim, size_t end, float theta);
 // x,out [H,S,D]; position_ids on device (u64) or, if null, pos0 + s.

@@ -7,9 +7,9 @@
 // from the logits wherever they are needed.  The reference draws one number from its PRNG per call (rng.float(f32));
 // that number is an argument here (u, or u_dev[step]), the generator stays with the caller.  Probabilities are formed
 // with the reference's operations in the reference's order per element (f32 divide by the temperature, subtract the
-// maximum, exp with the -88 cut-off, multiply by 1/sum); sums over the whole vocabulary are tree sums, so they can
-// differ from the reference's sequential sums in the last bits, which moves a boundary between two candidates by about
-// 1e-7 of the total.  The short sums top_k walks (at most 1024 candidates) are sequential in the reference's order.
+// maximum, exp with the -88 cut-off, multiply by 1/sum).  The reference's sums over the whole vocabulary are sequential
+// f32 loops (ops.zig:1585-1592, sampling.zig:139-147, 281-294, 200-214), and which candidate a draw lands on depends on
+// their rounding; seq_prefix below evaluates such a loop bit for bit with 1024 threads, so the index is the reference's.
 #pragma clang fp contract(off)
 #include "moon_internal.hpp"
 
@@ -23,6 +23,7 @@ constexpr int COPIES = 32;  // histogram copies, one per LDS bank, so that equal
 
 struct SampleArgs {
     const half_t *logits;
+    const float *logits_f32; // when set: the row as f32 (the type sampling.sample takes, sampling.zig:353); logits is unused
     int n, method, k;
     float temperature, min_p, u;
     float scale;        // 1 / temperature when that is exact (a power of two), else 0: the division is then a multiplication
@@ -43,7 +44,43 @@ struct SampleShared {
     unsigned sel[3];
     int first, last, result;
     unsigned count;
+    unsigned map0[16], map1[16]; // seq_prefix: the wavefronts' composed maps
+    float seq_s;                 // seq_prefix: the running sum at the start of chunk seq_cur
+    int seq_cross;
 };
+
+// exp of the sampling paths: the classic libm expf (k = round(x / ln 2), x - k ln2 in two parts, c = x - x^2 (P1 + x^2 P2),
+// 1 + (x c / (2 - c) - lo + hi), scaled by 2^k) spelled out in separate IEEE f32 operations (this file is compiled with
+// contraction off), because which candidate a draw lands on depends on the last bit of every term: the device and the
+// checker share this definition instead of each trusting its own library's expf.
+__device__ __forceinline__ float sampling_expf(float x) {
+    const float ln2hi = 6.9314575195e-1f, ln2lo = 1.4286067653e-6f, invln2 = 1.4426950216e+0f, P1 = 1.6666625440e-1f, P2 = -2.7667332906e-3f;
+    const unsigned ux = __float_as_uint(x);
+    const int sign = (int)(ux >> 31);
+    const unsigned hx = ux & 0x7fffffffu;
+    if (hx > 0x7f800000u) return x;
+    if (hx >= 0x42b17218u && !sign) return x * 0x1p127f;
+    if (sign && hx >= 0x42cff1b5u) return 0.0f;
+    float hi, lo, xr;
+    int k;
+    if (hx > 0x3eb17218u) {
+        if (hx > 0x3f851592u) k = (int)(invln2 * x + (sign ? -0.5f : 0.5f));
+        else k = 1 - sign - sign;
+        hi = x - (float)k * ln2hi;
+        lo = (float)k * ln2lo;
+        xr = hi - lo;
+    } else if (hx > 0x39000000u) {
+        k = 0;
+        hi = x;
+        lo = 0.0f;
+        xr = x;
+    } else
+        return 1.0f + x;
+    const float xx = xr * xr;
+    const float c = xr - xx * (P1 + xx * P2);
+    const float y = 1.0f + (__fdiv_rn(xr * c, 2.0f - c) - lo + hi);
+    return k == 0 ? y : ldexpf(y, k);
+}
 
 __device__ __forceinline__ float block_max(float v, float *s16) {
 #pragma unroll
@@ -79,59 +116,133 @@ __device__ __forceinline__ int block_min_int(int v, int *s16) {
     return r;
 }
 
+// A sequential f32 sum  s = 0; for i: s += w_i  over non-negative terms, evaluated bit for bit by the workgroup.
+// While s stays inside one binade [2^b, 2^(b+1)) it is an integer S in [2^23, 2^24) times ulp = 2^(b-23), and adding w
+// rounds S + w / ulp to an integer: S + E when the fraction of w / ulp is below a half, S + E + 1 when above, and to the
+// even one of the two on a tie.  So every term is a map S -> S + c[S & 1] with two small integers c[0], c[1]; such maps
+// compose associatively (the parity after the first map picks the second map's entry), which a scan over the 1024
+// threads' chunks evaluates exactly.  Nothing is trusted past the first chunk in which S would reach 2^24 (s leaves the
+// binade, the ulp changes) or a term is not smaller than the binade itself: the thread that owns that chunk runs the
+// plain float loop over it, and the next phase starts behind it with the new binade.  A sum crosses a few dozen binades
+// at most, most of them inside the first chunks.
+// each(f) calls f(i, w_i) for the thread's own indices in ascending order.  On return sh.scan[t] holds the running sum
+// BEFORE chunk t (exact), and the function returns the total.
+struct SeqMap {
+    unsigned c0, c1;
+};
+constexpr unsigned SEQ_BIG = 1u << 24, SEQ_CAP = 1u << 26;
+__device__ __forceinline__ SeqMap seq_compose(SeqMap a, SeqMap b) { // a first, then b
+    SeqMap r;
+    r.c0 = min(a.c0 + ((a.c0 & 1u) ? b.c1 : b.c0), SEQ_CAP);
+    r.c1 = min(a.c1 + (((1u + a.c1) & 1u) ? b.c1 : b.c0), SEQ_CAP);
+    return r;
+}
+// sb: biased exponent of the running sum, 0 when the sum is zero or below the second normal binade (then every non-zero
+// term ends the phase)
+__device__ __forceinline__ SeqMap seq_elem(float w, int sb) {
+    const unsigned bits = __float_as_uint(w);
+    if ((bits << 1) == 0u) return SeqMap{0u, 0u};
+    if (sb == 0) return SeqMap{SEQ_BIG, SEQ_BIG};
+    int eb = (int)((bits >> 23) & 255u);
+    unsigned em = bits & 0x7fffffu;
+    if (eb == 0) eb = 1; // subnormal: no implicit bit
+    else em |= 0x800000u;
+    const int k = sb - eb; // w / ulp = em / 2^k
+    if (k <= 0) return SeqMap{SEQ_BIG, SEQ_BIG};
+    if (k >= 25) return SeqMap{0u, 0u};
+    const unsigned E = k >= 24 ? 0u : em >> k, rem = em & ((1u << k) - 1u), half = 1u << (k - 1);
+    if (rem < half) return SeqMap{E, E};
+    if (rem > half) return SeqMap{E + 1u, E + 1u};
+    return SeqMap{E + (E & 1u), E + ((E + 1u) & 1u)}; // tie: to the even neighbour
+}
+template <class Each>
+__device__ __forceinline__ float seq_prefix(Each each, SampleShared &sh) {
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    __syncthreads();
+    if (t == 0) sh.seq_s = 0.f;
+    int cur = 0; // chunks before cur are done: sh.scan[0..cur] are final
+    __syncthreads();
+    while (cur < ST) {
+        const float s = sh.seq_s;
+        const unsigned sbits = __float_as_uint(s);
+        int sb = (int)((sbits >> 23) & 255u);
+        if (sb <= 1) sb = 0;
+        const unsigned S0 = sb ? ((sbits & 0x7fffffu) | 0x800000u) : 0u;
+        SeqMap m{0u, 0u};
+        if (t >= cur) each([&](int, float w) { m = seq_compose(m, seq_elem(w, sb)); });
+        SeqMap inc = m; // inclusive scan over the threads in ascending order
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            SeqMap o;
+            o.c0 = __shfl_up(inc.c0, off, 64);
+            o.c1 = __shfl_up(inc.c1, off, 64);
+            if (lane >= off) inc = seq_compose(o, inc);
+        }
+        if (lane == 63) {
+            sh.map0[wave] = inc.c0;
+            sh.map1[wave] = inc.c1;
+        }
+        if (t == 0) sh.seq_cross = ST;
+        __syncthreads();
+        SeqMap before{0u, 0u};
+        for (int w = 0; w < wave; w++) before = seq_compose(before, SeqMap{sh.map0[w], sh.map1[w]});
+        inc = seq_compose(before, inc);
+        SeqMap exc; // everything before this thread's chunk
+        exc.c0 = __shfl_up(inc.c0, 1, 64);
+        exc.c1 = __shfl_up(inc.c1, 1, 64);
+        if (lane == 0) exc = before;
+        const unsigned p = S0 & 1u;
+        const unsigned start = S0 + (p ? exc.c1 : exc.c0), end = S0 + (p ? inc.c1 : inc.c0);
+        // sb == 0: S counts nothing, a non-zero term anywhere in the chunk shows as >= SEQ_BIG
+        const bool crossed = end >= SEQ_BIG;
+        if (t >= cur && crossed) atomicMin(&sh.seq_cross, t);
+        __syncthreads();
+        const int x = sh.seq_cross;
+        if (t >= cur && t <= x && t < ST) sh.scan[t] = sb ? __uint_as_float(((unsigned)sb << 23) | (start & 0x7fffffu)) : s;
+        if (x == ST) {
+            if (t == ST - 1) sh.seq_s = sb ? __uint_as_float(((unsigned)sb << 23) | (end & 0x7fffffu)) : s;
+            cur = ST;
+        } else {
+            if (t == x) { // the plain loop over the chunk that leaves the binade
+                float v = sh.scan[t];
+                each([&](int, float w) { v += w; });
+                sh.seq_s = v;
+            }
+            cur = x + 1;
+        }
+        __syncthreads();
+    }
+    return sh.seq_s;
+}
+
 // The candidate walk of multinomial_sampling / min_p_sampling (sampling.zig:276-297, 199-218): candidates in index
-// order with weight wt(probability) (0 = not a candidate), r = u * (sum of the weights), first candidate with
-// r < running sum.  each(f) calls f(i, probability) for the thread's own indices in ascending order.  Sequential sums
-// inside a chunk, a scan over the 1024 chunk sums, then only the chunk that holds r is walked.  A chunk is only named if
-// it has a candidate, and inside it the last candidate stands in when rounding leaves r at or above the chunk's own
-// running sum (the scan adds in another order), so the result is always a candidate next to r.  Returns -1 when r is
-// not below the total (the caller's fall-back), which for u close to 1 depends on how u * total rounds, as it does in
-// the reference.
+// order with weight wt(probability) (0 = not a candidate; adding 0 changes nothing, so skipping them is the same loop),
+// r = u * (sum of the weights), first candidate with r < running sum.  each(f) calls f(i, probability) for the thread's
+// own indices in ascending order.  The running sums at the chunk starts and the total are the reference's bits
+// (seq_prefix); the one chunk whose end is the first above r is walked with the same float additions.  Returns -1 when r
+// is not below the total (the caller's fall-back).
 template <class Each, class Wt>
 __device__ __forceinline__ int walk_in_index_order(Each each, Wt wt, float u, SampleShared &sh) {
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    float cs = 0.f;
-    each([&](int, float pi) { cs += wt(pi); });
-    float incl = cs;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float o = __shfl_up(incl, off, 64);
-        if (lane >= off) incl += o;
-    }
-    __syncthreads();
-    if (lane == 63) sh.s16[wave] = incl;
-    if (t == 0) {
-        sh.first = ST;
-        sh.last = -1;
-    }
-    __syncthreads();
-    float base = 0.f, total = 0.f;
-    for (int wv = 0; wv < ST / 64; wv++) {
-        if (wv == wave) base = total;
-        total += sh.s16[wv];
-    }
-    incl = base + incl;
-    sh.scan[t] = incl;
+    const int t = threadIdx.x;
+    const float total = seq_prefix([&](auto f) { each([&](int i, float pi) { f(i, wt(pi)); }); }, sh);
     const float r = u * total;
-    if (cs > 0.f && r < incl) atomicMin(&sh.first, t);
-    if (cs > 0.f) atomicMax(&sh.last, t);
+    if (t == 0) sh.first = ST;
     __syncthreads();
-    int c = sh.first;
-    // r below the total but not below any chunk's running sum (the scan's sums are not exactly monotone): the last candidate
-    if (c == ST && r < total) c = sh.last;
-    if (c == ST || c < 0) return -1;
-    if (t == c) { // walk this chunk from the running sum the chunk before it ended on
-        float cum = c ? sh.scan[c - 1] : 0.f;
-        int res = -1, last = -1;
+    const float end = t + 1 < ST ? sh.scan[t + 1] : total; // the running sum behind this chunk
+    if (r < end) atomicMin(&sh.first, t);
+    __syncthreads();
+    const int c = sh.first;
+    if (c == ST) return -1;
+    if (t == c) {
+        float cum = sh.scan[c];
+        int res = -1;
         each([&](int i, float pi) {
-            const float w = wt(pi);
             if (res < 0) {
-                cum += w;
-                if (w > 0.f) last = i;
-                if (w > 0.f && r < cum) res = i;
+                cum += wt(pi);
+                if (r < cum) res = i;
             }
         });
-        sh.result = res >= 0 ? res : last;
+        sh.result = res;
     }
     __syncthreads();
     return sh.result;
@@ -288,6 +399,8 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs p) {
     SampleShared &sh = *reinterpret_cast<SampleShared *>(dyn_lds);
     const int t = threadIdx.x, n = p.n;
     const half_t *__restrict__ logits = p.logits;
+    const float *__restrict__ logits_f32 = p.logits_f32;
+    auto lg = [&](int i) { return logits_f32 ? logits_f32[i] : (float)logits[i]; };
     const float temperature = p.temperature;
     const float u = p.u_dev ? p.u_dev[p.state ? p.state[1] : 0] : p.u;
     const int C = J ? J : (n + ST - 1) / ST, lo = min(n, t * C), hi = min(n, lo + C); // the J == 0 kernel's chunk
@@ -327,26 +440,30 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs p) {
         }
         __syncthreads(); // sh lives in the same memory
     } else {
-        for (int i = lo; i < hi; i++) mx = fmaxf(mx, (float)logits[i]);
+        for (int i = lo; i < hi; i++) mx = fmaxf(mx, lg(i));
     }
     mx = x_of(block_max(mx, sh.s16));
     auto e_of = [&](float logit) {
         const float d = x_of(logit) - mx;
-        return d > -88.0f ? expf(d) : 0.f; // ops.zig:1589-1590, sampling.zig:145
+        return d > -88.0f ? sampling_expf(d) : 0.f; // ops.zig:1589-1590, sampling.zig:145
     };
-    float sum = 0.f;
     if constexpr (J > 0) {
 #pragma unroll
-        for (int j = 0; j < J; j++) {
-            v[j] = e_of(v[j]);
-            sum += v[j];
-        }
-    } else {
-        for (int i = lo; i < hi; i++) sum += e_of((float)logits[i]);
+        for (int j = 0; j < J; j++) v[j] = e_of(v[j]);
     }
-    sum = block_sum(sum, sh.s16);
+    // the sum of the exps in the reference's sequential order (ops.zig:1585-1592; sampling.zig:139-147 for min_p)
+    const float sum = seq_prefix(
+        [&](auto f) {
+            if constexpr (J > 0) {
+#pragma unroll
+                for (int j = 0; j < J; j++) f(t * J + j, v[j]);
+            } else {
+                for (int i = lo; i < hi; i++) f(i, e_of(lg(i)));
+            }
+        },
+        sh);
     const float inv_sum = __fdiv_rn(1.0f, sum);
-    const bool normalise = METHOD == MOON_SAMPLE_MIN_P || sum > 0.f; // ops.softmax leaves the exps alone when their sum is not positive
+    const bool normalise = METHOD == MOON_SAMPLE_MIN_P || sum > 0.f; // ops.softmax normalises only a positive sum (ops.zig:1595; otherwise it leaves its input, the scaled logits, in place: only a not-a-number logit gets there, and the exps stand in here)
     if constexpr (J > 0) {
         if (normalise) {
 #pragma unroll
@@ -362,7 +479,7 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs p) {
             for (int j = 0; j < J; j++) f(first + j, v[j]);
         } else {
             for (int i = lo; i < hi; i++) {
-                const float e = e_of((float)logits[i]);
+                const float e = e_of(lg(i));
                 f(i, normalise ? e * inv_sum : e);
             }
         }
@@ -431,7 +548,7 @@ hipError_t launch_sample_kernel(hipStream_t stream, const SampleArgs &a) {
 
 // sampling.sample for methods multinomial / top_k / min_p; greedy goes to the arg-max kernels (it ignores the temperature).
 int launch_sample(moon_ctx *ctx, const half_t *logits, size_t n, const moon_sampling_config *cfg, float u, const float *u_dev,
-                  uint32_t *state, uint32_t *out_ids, uint32_t *out, uint32_t bump_pos) {
+                  uint32_t *state, uint32_t *out_ids, uint32_t *out, uint32_t bump_pos, const float *logits_f32) {
     if (!cfg) return moon_fail(ctx, MOON_EINVAL, "sample: null config");
     if (!n || n > 0x3fffffff) return moon_fail(ctx, MOON_EINVAL, "sample: empty or oversized tensor");
     if (cfg->method < MOON_SAMPLE_MULTINOMIAL || cfg->method > MOON_SAMPLE_MIN_P)
@@ -445,13 +562,13 @@ int launch_sample(moon_ctx *ctx, const half_t *logits, size_t n, const moon_samp
         if (k > (size_t)ST) return moon_fail(ctx, MOON_EINVAL, "sample: top_k %zu (at most %d candidates are sorted on the device)", k, ST);
     }
     SampleArgs a;
-    a.logits = logits; a.n = (int)n; a.method = cfg->method; a.k = (int)k;
+    a.logits = logits; a.logits_f32 = logits_f32; a.n = (int)n; a.method = cfg->method; a.k = (int)k;
     a.temperature = cfg->temperature; a.min_p = cfg->min_p; a.u = u; a.u_dev = u_dev;
     int exponent = 0;
     a.scale = (std::frexp(cfg->temperature, &exponent) == 0.5f && exponent > -100 && exponent < 100) ? 1.0f / cfg->temperature : 0.f;
     a.state = state; a.out_ids = out_ids; a.out = out; a.bump_pos = bump_pos;
     const size_t per_thread = (n + ST - 1) / ST;
-    const bool in_registers = per_thread <= 64 && (reinterpret_cast<uintptr_t>(logits) & 3) == 0;
+    const bool in_registers = !logits_f32 && per_thread <= 64 && (reinterpret_cast<uintptr_t>(logits) & 3) == 0;
     hipError_t e;
     if (!in_registers) e = launch_sample_kernel<0>(ctx->stream, a);
     else if (per_thread <= 4) e = launch_sample_kernel<4>(ctx->stream, a);

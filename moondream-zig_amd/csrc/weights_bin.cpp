@@ -137,9 +137,16 @@ extern "C" int moon_bin_open(const char *path, moon_bin **out, char *err, size_t
             pos += 8;
             if (d > (uint64_t(1) << 40)) return bail(bin_fail(err, err_len, MOON_EFORMAT, "moondream.bin: tensor '%s': dimension too large", t.name.c_str()));
             t.dims[i] = (size_t)d;
+            // four dimensions of up to 2^40 each would wrap the product: nothing larger than the file can be meant
+            if (d && t.numel > bin->size / (size_t)d)
+                return bail(bin_fail(err, err_len, MOON_EFORMAT, "moondream.bin: tensor '%s': %u dimensions multiply to more elements than the file has bytes (InvalidRead)",
+                                     t.name.c_str(), ndim));
             t.numel *= (size_t)d;
         }
-        (void)numel32; // the reader trusts the dims, as the reference does (weights.zig:183-187); the count wraps at 2^32 for no tensor here
+        // the record's own element count (a u32, weights.zig:58) has to agree with the dimensions, modulo its 32 bits
+        if (numel32 != (uint32_t)t.numel)
+            return bail(bin_fail(err, err_len, MOON_EFORMAT, "moondream.bin: tensor '%s': header says %u elements, the dimensions %zu (InvalidHeader)",
+                                 t.name.c_str(), numel32, t.numel));
         if (!known_name(t.name)) return bail(bin_fail(err, err_len, MOON_EFORMAT, "moondream.bin: unknown tensor '%s' (UnknownTensorName)", t.name.c_str()));
         if ((bin->size - pos) / 2 < t.numel)
             return bail(bin_fail(err, err_len, MOON_EFORMAT, "moondream.bin: tensor '%s' needs %zu bytes, file ends after %zu (InvalidRead)", t.name.c_str(),

@@ -5,6 +5,8 @@ from __future__ import annotations
 
 import ctypes as C
 
+import numpy as np
+
 from . import _lib as L
 from .context import Context, default_context, f16, ptr
 
@@ -32,6 +34,25 @@ def sample(logits, config: L.SamplingConfig, u: float = 0.0, ctx: Context | None
     logits = f16(logits).reshape(-1)
     idx = C.c_size_t()
     ctx.check(ctx.lib.moon_sample(ctx.handle, ptr(logits), logits.size, C.byref(config), u, C.byref(idx)))
+    return int(idx.value)
+
+
+def sample_f32(logits, config: L.SamplingConfig, u: float = 0.0, ctx: Context | None = None) -> int:
+    """sampling.sample(tensor: *Tensor(f32), config, rng, allocator) (sampling.zig:353-389) on the f32 row the reference
+    hands it (moondream.zig:335-337)."""
+    ctx = ctx or default_context()
+    logits = np.ascontiguousarray(logits, dtype=np.float32).reshape(-1)
+    idx = C.c_size_t()
+    ctx.check(ctx.lib.moon_sample_f32(ctx.handle, logits.ctypes.data_as(C.c_void_p), logits.size, C.byref(config), u, C.byref(idx)))
+    return int(idx.value)
+
+
+def argmax_f32(logits, ctx: Context | None = None) -> int:
+    """sampling.argmax(f32, tensor) (sampling.zig:257-273)."""
+    ctx = ctx or default_context()
+    logits = np.ascontiguousarray(logits, dtype=np.float32).reshape(-1)
+    idx = C.c_size_t()
+    ctx.check(ctx.lib.moon_argmax_f32(ctx.handle, logits.ctypes.data_as(C.c_void_p), logits.size, C.byref(idx)))
     return int(idx.value)
 
 

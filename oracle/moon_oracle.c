@@ -403,6 +403,60 @@ size_t orc_argmax_f16(const orc_f16 *logits, size_t n) {
 }
 
 /* ------------------------------------------------------------------ sampling (sampling.zig) */
+/* exp for the sampling paths.  The reference's @exp(f32) comes from its language runtime's libm port (the classic
+ * expf: k = round(x / ln 2), x - k ln2 in two parts, c = x - x^2 (P1 + x^2 P2), 1 + (x c / (2 - c) - lo + hi), scaled
+ * by 2^k); which candidate a draw lands on depends on the last bit of every term, so the checker and the device share
+ * this one definition, evaluated with separate IEEE f32 operations, instead of each trusting its own library's expf. */
+static float orc_expf_sampling(float x) {
+    static const float ln2hi = 6.9314575195e-1f, ln2lo = 1.4286067653e-6f, invln2 = 1.4426950216e+0f, P1 = 1.6666625440e-1f,
+                       P2 = -2.7667332906e-3f;
+    union { float f; uint32_t u; } w;
+    w.f = x;
+    const int sign = (int)(w.u >> 31);
+    const uint32_t hx = w.u & 0x7fffffffu;
+    if (hx > 0x7f800000u) return x;                       /* NaN */
+    if (hx >= 0x42b17218u && !sign) return x * 0x1p127f;  /* overflow */
+    if (sign && hx >= 0x42cff1b5u) return 0.0f;           /* underflow */
+    volatile float hi, lo, xr;
+    int k;
+    if (hx > 0x3eb17218u) {                               /* |x| > 0.5 ln2 */
+        if (hx > 0x3f851592u) {                           /* |x| > 1.5 ln2 */
+            volatile float kf = invln2 * x;
+            kf = kf + (sign ? -0.5f : 0.5f);
+            k = (int)kf;
+        } else
+            k = 1 - sign - sign;
+        volatile float t1 = (float)k * ln2hi;
+        hi = x - t1;
+        lo = (float)k * ln2lo;
+        xr = hi - lo;
+    } else if (hx > 0x39000000u) {                        /* |x| > 2^-14 */
+        k = 0;
+        hi = x;
+        lo = 0.0f;
+        xr = x;
+    } else
+        return 1.0f + x;
+    volatile float xx = xr * xr;
+    volatile float p = xx * P2;
+    p = P1 + p;
+    p = xx * p;
+    volatile float c = xr - p;
+    volatile float num = xr * c;
+    volatile float den = 2.0f - c;
+    volatile float q = num / den;
+    q = q - lo;
+    q = q + hi;
+    volatile float y = 1.0f + q;
+    if (k == 0) return y;
+    return ldexpf(y, k);
+}
+
+/* orc_expf_sampling over an array (for the tests that pin it) */
+void orc_sampling_expf(const float *x, float *y, size_t n) {
+    for (size_t i = 0; i < n; i++) y[i] = orc_expf_sampling(x[i]);
+}
+
 /* ops.softmax over one f32 row (ops.zig:1574-1601): running maximum, exp with the -88 cut-off, sequential sum,
  * multiply by 1/sum when the sum is positive. */
 static void sample_softmax(float *x, size_t n) {
@@ -412,7 +466,7 @@ static void sample_softmax(float *x, size_t n) {
     float sum = 0.f;
     for (size_t i = 0; i < n; i++) {
         const float val = x[i] - max;
-        x[i] = val > -88.0f ? expf(val) : 0.f;
+        x[i] = val > -88.0f ? orc_expf_sampling(val) : 0.f;
         sum += x[i];
     }
     if (sum > 0.f) {
@@ -439,16 +493,30 @@ static void sample_sort_desc(size_t *idx, size_t *tmp, const float *p, size_t n)
  * draws from its PRNG (rng.float(f32), in [0,1)) passed in as u.  method: 0 greedy, 1 multinomial, 2 top_k, 3 min_p.
  * Returns 0, or 1 InvalidTemperature (sampling.zig:344), 2 a top_k of 0 (the reference indexes [k-1] of an empty
  * slice there), 3 unknown method / empty input. */
+int orc_sample_f32(const float *logits, size_t n, int method, float temperature, size_t top_k, float min_p, float u, size_t *index);
 int orc_sample_f16(const orc_f16 *logits, size_t n, int method, float temperature, size_t top_k, float min_p, float u, size_t *index) {
+    if (!n) return 3;
+    float *x = (float *)malloc(n * sizeof(float)); /* moondream.zig:335: logits.castWithSimd(f32) */
+    for (size_t i = 0; i < n; i++) x[i] = orc_h2f(logits[i]);
+    const int rc = orc_sample_f32(x, n, method, temperature, top_k, min_p, u, index);
+    free(x);
+    return rc;
+}
+/* the same on the f32 row sampling.sample takes (sampling.zig:353-358) */
+int orc_sample_f32(const float *logits, size_t n, int method, float temperature, size_t top_k, float min_p, float u, size_t *index) {
     if (!n || method < 0 || method > 3) return 3;
-    if (method == 0) { /* sampling.zig:370-372: temperature is not applied */
-        *index = orc_argmax_f16(logits, n);
+    if (method == 0) { /* sampling.zig:370-372: temperature is not applied; argmax: strict >, first maximum wins (:257-273) */
+        size_t idx = 0;
+        float best = logits[0];
+        for (size_t i = 0; i < n; i++)
+            if (logits[i] > best) { best = logits[i]; idx = i; }
+        *index = idx;
         return 0;
     }
     if (temperature != 1.0f && !(temperature > 0.f)) return 1;
     if (method == 2 && top_k == 0) return 2;
     float *x = (float *)malloc(n * sizeof(float));
-    for (size_t i = 0; i < n; i++) x[i] = orc_h2f(logits[i]);
+    for (size_t i = 0; i < n; i++) x[i] = logits[i];
     if (temperature != 1.0f)
         for (size_t i = 0; i < n; i++) x[i] = x[i] / temperature; /* sampling.zig:347-349 */
     int rc = 0;
@@ -485,7 +553,7 @@ int orc_sample_f16(const orc_f16 *logits, size_t n, int method, float temperatur
         float sum = 0.f;
         for (size_t i = 0; i < n; i++) {
             const float d = x[i] - max_logit;
-            x[i] = d > -88.0f ? expf(d) : 0.f;
+            x[i] = d > -88.0f ? orc_expf_sampling(d) : 0.f;
             sum += x[i];
         }
         const float inv_sum = 1.0f / sum;

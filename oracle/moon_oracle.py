@@ -54,6 +54,8 @@ def _load():
         "orc_merge_heads": (None, [vp, vp, sz, sz, sz]),
         "orc_argmax_f16": (sz, [vp, sz]),
         "orc_sample_f16": (C.c_int, [vp, sz, C.c_int, f32, sz, f32, f32, C.POINTER(sz)]),
+        "orc_sample_f32": (C.c_int, [vp, sz, C.c_int, f32, sz, f32, f32, C.POINTER(sz)]),
+        "orc_sampling_expf": (None, [vp, vp, sz]),
         "orc_rel_frobenius": (C.c_double, [vp, vp, sz]),
         "orc_refstyle_gemv_nt": (None, [vp, vp, vp, sz, sz, C.c_int]),
         "orc_refstyle_hgemm": (None, [vp, vp, vp, sz, sz, sz, C.c_int, C.c_int]),
@@ -284,6 +286,24 @@ def sample(logits, method: str, u: float, temperature: float = 0.5, top_k: int =
     if rc:
         raise ValueError({1: "InvalidTemperature", 2: "top_k of 0", 3: "empty input or unknown method"}[rc])
     return int(idx.value)
+
+
+def sample_f32(logits, method: str, u: float, temperature: float = 0.5, top_k: int = 3, min_p: float = 0.05) -> int:
+    """sampling.sample on the f32 row it takes in the reference (sampling.zig:353-358)."""
+    logits = np.ascontiguousarray(logits, dtype=np.float32).reshape(-1)
+    idx = C.c_size_t(0)
+    rc = _lib.orc_sample_f32(_p(logits), logits.size, SAMPLING_METHODS[method], temperature, top_k, min_p, u, C.byref(idx))
+    if rc:
+        raise ValueError({1: "InvalidTemperature", 2: "top_k of 0", 3: "empty input or unknown method"}[rc])
+    return int(idx.value)
+
+
+def sampling_expf(x):
+    """The exp the sampling paths use (one definition shared with the device), element-wise on f32."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    y = np.empty_like(x)
+    _lib.orc_sampling_expf(_p(x), _p(y), x.size)
+    return y
 
 
 def rel_frobenius(a, b) -> float:

@@ -144,3 +144,30 @@ def test_registered_weight_is_reused(moon, O, ctx):
     assert O.rel_frobenius(y1, ref) <= TOL and np.array_equal(y1, y2)
     assert np.all(y3 == 0)
     w[:] = keep
+
+
+def test_registered_weight_in_hgemm_layout(moon, O, ctx):
+    """hgemm.matmul reads B as [K, N] (hgemm.zig:210-216).  A registered weight used that way gets its [N, K] copy once, on
+    the first call; later calls (also with another row count, and as a one-row product) use it and give the bits of the
+    unregistered path, and a weight registered again takes its new contents."""
+    a = O.fill_normal_f16((729, 1152), 0, 0, 1.0)
+    w = O.fill_normal_f16((1152, 776), 0, 1, 0.02)  # [K, N]
+    plain = moon.hgemm.matmul(a, w, ctx=ctx)
+    assert O.rel_frobenius(plain, O.hgemm(a, w)) <= TOL
+    ctx.register_weight(w)
+    first = moon.hgemm.matmul(a, w, ctx=ctx)
+    keep = w.copy()
+    w[:] = 0  # the resident copies are what is multiplied now
+    again = moon.hgemm.matmul(a, w, ctx=ctx)
+    fewer = moon.hgemm.matmul(a[:33], w, ctx=ctx)
+    one = moon.hgemm.matmul(a[:1], w, ctx=ctx)
+    w[:] = keep
+    assert np.array_equal(first, plain) and np.array_equal(again, plain)
+    assert np.array_equal(fewer, moon.hgemm.matmul(a[:33], keep, ctx=ctx))
+    assert O.rel_frobenius(one, O.hgemm(a[:1], keep)) <= TOL
+    w[:] = keep * np.float16(2)
+    ctx.register_weight(w)  # again: both resident copies are replaced
+    doubled = moon.hgemm.matmul(a, w, ctx=ctx)
+    ctx.unregister_weight(w)
+    assert O.rel_frobenius(doubled, O.hgemm(a, w)) <= TOL
+    assert np.array_equal(moon.hgemm.matmul(a, w, ctx=ctx), doubled)

@@ -486,3 +486,15 @@ def test_image_patches_values_and_layout(O):
             assert got[b, t, col] == lut[img[y, x, c]]
     with pytest.raises(ValueError, match="InvalidPatchSize"):
         O.image_patches(np.zeros((15, 14, 3), dtype=np.uint8), 14)
+
+
+def test_sampling_expf_against_float64(O):
+    """The exp the sampling paths share with the device (the classic two-part-reduction expf, error below one ulp): pinned
+    against numpy's float64 exp over the range the -88 cut-off leaves, at the reduction's branch points and at 0."""
+    x = np.concatenate([np.linspace(-88, 0, 200001), -np.logspace(-8, 1.9, 50000),
+                        [0.0, -0.0, -87.999, -1e-5, -0.3465, -0.3466, -1.0397, -1.0398, -6.1e-5, -6.2e-5]]).astype(np.float32)
+    y = O.sampling_expf(x)
+    ref = np.exp(x.astype(np.float64))
+    ulp = np.spacing(np.maximum(ref, 2.0 ** -126).astype(np.float32)).astype(np.float64)
+    assert np.max(np.abs(y.astype(np.float64) - ref) / ulp) < 1.0
+    assert O.sampling_expf(np.float32([0.0]))[0] == 1.0

@@ -75,6 +75,10 @@ HDR = struct.pack("<II", 0x4D4F4F4E, 2)
     (HDR + struct.pack("<III", 6, 1, 4) + b"t_ln_w" + struct.pack("<Q", 4) + b"\x00" * 6, "InvalidRead"),
     (HDR + struct.pack("<III", 5, 1, 1) + b"bogus" + struct.pack("<Q", 1) + b"\x00\x00", "UnknownTensorName"),
     (b"MOO", "InvalidRead"),
+    # the record's element count disagrees with its dimensions
+    (HDR + struct.pack("<III", 6, 1, 3) + b"t_ln_w" + struct.pack("<Q", 4) + b"\x00" * 8, "InvalidHeader"),
+    # four dimensions whose product wraps 64 bits to a small number (2^20 each: 2^80 -> 0 elements, "fits" any file)
+    (HDR + struct.pack("<III", 6, 4, 0) + b"t_ln_w" + struct.pack("<4Q", 1 << 20, 1 << 20, 1 << 20, 1 << 20) + b"\x00" * 64, "InvalidRead"),
 ])
 def test_malformed_files_are_rejected_like_the_reference(moon, tmp_path, payload, text):
     path = _write(tmp_path / "bad.bin", payload)
