@@ -10,11 +10,16 @@
 // maximum, exp with the -88 cut-off, multiply by 1/sum).  The reference's sums over the whole vocabulary are sequential
 // f32 loops (ops.zig:1585-1592, sampling.zig:139-147, 281-294, 200-214), and which candidate a draw lands on depends on
 // their rounding; seq_prefix below evaluates such a loop bit for bit with 1024 threads, so the index is the reference's.
+// That evaluation costs a few hundred microseconds, so the kernel first takes its sums the fast way and keeps the answer
+// only where it provably cannot depend on how they were rounded (the draw clear of the running sums next to it by more
+// than any evaluation can move them, the candidate set clear of its thresholds); otherwise it runs the exact one.  With
+// the reference's default (top_k 3) the exact path is taken about once in 10^5 draws.
 #pragma clang fp contract(off)
 #include "moon_internal.hpp"
 
 #include <atomic>
 #include <cmath>
+#include <type_traits>
 
 namespace {
 
@@ -47,6 +52,7 @@ struct SampleShared {
     unsigned map0[16], map1[16]; // seq_prefix: the wavefronts' composed maps
     float seq_s;                 // seq_prefix: the running sum at the start of chunk seq_cur
     int seq_cross;
+    int safe;                    // the quick path's result is provably the exact path's
 };
 
 // exp of the sampling paths: the classic libm expf (k = round(x / ln 2), x - k ln2 in two parts, c = x - x^2 (P1 + x^2 P2),
@@ -138,29 +144,30 @@ __device__ __forceinline__ SeqMap seq_compose(SeqMap a, SeqMap b) { // a first, 
     return r;
 }
 // sb: biased exponent of the running sum, 0 when the sum is zero or below the second normal binade (then every non-zero
-// term ends the phase)
+// term ends the phase).  Branch-free: this runs for every term in every phase.
 __device__ __forceinline__ SeqMap seq_elem(float w, int sb) {
     const unsigned bits = __float_as_uint(w);
-    if ((bits << 1) == 0u) return SeqMap{0u, 0u};
-    if (sb == 0) return SeqMap{SEQ_BIG, SEQ_BIG};
-    int eb = (int)((bits >> 23) & 255u);
-    unsigned em = bits & 0x7fffffu;
-    if (eb == 0) eb = 1; // subnormal: no implicit bit
-    else em |= 0x800000u;
-    const int k = sb - eb; // w / ulp = em / 2^k
-    if (k <= 0) return SeqMap{SEQ_BIG, SEQ_BIG};
-    if (k >= 25) return SeqMap{0u, 0u};
-    const unsigned E = k >= 24 ? 0u : em >> k, rem = em & ((1u << k) - 1u), half = 1u << (k - 1);
-    if (rem < half) return SeqMap{E, E};
-    if (rem > half) return SeqMap{E + 1u, E + 1u};
-    return SeqMap{E + (E & 1u), E + ((E + 1u) & 1u)}; // tie: to the even neighbour
+    const unsigned ebf = (bits >> 23) & 255u;
+    const unsigned em = (bits & 0x7fffffu) | (ebf ? 0x800000u : 0u); // subnormal: no implicit bit, exponent as for 1
+    const int k = sb - (int)(ebf ? ebf : 1u);                        // w / ulp = em / 2^k
+    const unsigned kc = (unsigned)min(max(k, 1), 25);
+    const unsigned E = em >> kc, frac = em & ((1u << kc) - 1u), half = 1u << (kc - 1u); // em < 2^24: E is 0 from k = 24 on
+    const unsigned up = frac > half ? 1u : 0u, tie = frac == half ? 1u : 0u;
+    SeqMap m{E + up + (tie & E), E + up + (tie & ~E)}; // tie: to the even neighbour, which depends on the parity of S + E
+    const bool zero = (bits << 1) == 0u;
+    const bool big = !zero && (sb == 0 || k <= 0); // no binade to count in, or a term not smaller than the binade itself
+    m.c0 = zero ? 0u : big ? SEQ_BIG : m.c0;
+    m.c1 = zero ? 0u : big ? SEQ_BIG : m.c1;
+    return m;
 }
 template <class Each>
 __device__ __forceinline__ float seq_prefix(Each each, SampleShared &sh) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     __syncthreads();
     if (t == 0) sh.seq_s = 0.f;
-    int cur = 0; // chunks before cur are done: sh.scan[0..cur] are final
+    int cur = 0;  // chunks before cur are done: sh.scan[0..cur) are final
+    int win = 64; // chunks looked at per phase: doubled whenever a phase ends without leaving its binade, so that the terms
+                  // are visited two or three times in all rather than once per binade
     __syncthreads();
     while (cur < ST) {
         const float s = sh.seq_s;
@@ -168,8 +175,13 @@ __device__ __forceinline__ float seq_prefix(Each each, SampleShared &sh) {
         int sb = (int)((sbits >> 23) & 255u);
         if (sb <= 1) sb = 0;
         const unsigned S0 = sb ? ((sbits & 0x7fffffu) | 0x800000u) : 0u;
+        const int wend = min(cur + win, ST);
+        const bool mine = t >= cur && t < wend;
         SeqMap m{0u, 0u};
-        if (t >= cur) each([&](int, float w) { m = seq_compose(m, seq_elem(w, sb)); });
+        if (mine)
+            each([&](int, float w) {
+                m = seq_compose(m, seq_elem(w, sb));
+            });
         SeqMap inc = m; // inclusive scan over the threads in ascending order
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
@@ -194,14 +206,14 @@ __device__ __forceinline__ float seq_prefix(Each each, SampleShared &sh) {
         const unsigned p = S0 & 1u;
         const unsigned start = S0 + (p ? exc.c1 : exc.c0), end = S0 + (p ? inc.c1 : inc.c0);
         // sb == 0: S counts nothing, a non-zero term anywhere in the chunk shows as >= SEQ_BIG
-        const bool crossed = end >= SEQ_BIG;
-        if (t >= cur && crossed) atomicMin(&sh.seq_cross, t);
+        if (mine && end >= SEQ_BIG) atomicMin(&sh.seq_cross, t);
         __syncthreads();
         const int x = sh.seq_cross;
-        if (t >= cur && t <= x && t < ST) sh.scan[t] = sb ? __uint_as_float(((unsigned)sb << 23) | (start & 0x7fffffu)) : s;
-        if (x == ST) {
-            if (t == ST - 1) sh.seq_s = sb ? __uint_as_float(((unsigned)sb << 23) | (end & 0x7fffffu)) : s;
-            cur = ST;
+        if (mine && t <= x) sh.scan[t] = sb ? __uint_as_float(((unsigned)sb << 23) | (start & 0x7fffffu)) : s;
+        if (x == ST) { // the window stayed inside the binade
+            if (t == wend - 1) sh.seq_s = sb ? __uint_as_float(((unsigned)sb << 23) | (end & 0x7fffffu)) : s;
+            cur = wend;
+            win = min(2 * win, ST);
         } else {
             if (t == x) { // the plain loop over the chunk that leaves the binade
                 float v = sh.scan[t];
@@ -222,7 +234,7 @@ __device__ __forceinline__ float seq_prefix(Each each, SampleShared &sh) {
 // (seq_prefix); the one chunk whose end is the first above r is walked with the same float additions.  Returns -1 when r
 // is not below the total (the caller's fall-back).
 template <class Each, class Wt>
-__device__ __forceinline__ int walk_in_index_order(Each each, Wt wt, float u, SampleShared &sh) {
+__device__ __forceinline__ int walk_exact(Each each, Wt wt, float u, SampleShared &sh) {
     const int t = threadIdx.x;
     const float total = seq_prefix([&](auto f) { each([&](int i, float pi) { f(i, wt(pi)); }); }, sh);
     const float r = u * total;
@@ -248,15 +260,80 @@ __device__ __forceinline__ int walk_in_index_order(Each each, Wt wt, float u, Sa
     return sh.result;
 }
 
+// The quick form of the same walk: sequential sums inside a chunk, a scan over the 1024 chunk sums, the chunk that holds
+// r walked by one thread.  Its sums are not the reference's bits, so it only answers when the answer cannot depend on them:
+// with m candidates, the running sums and r = u * total, taken in any order and with any 1 / sum behind the probabilities
+// (every probability is one multiplication by the same factor, so the factor cancels in r against a running sum up to the
+// roundings), stay within (6 m + 32) 2^-24 of the total of their exact values; if r keeps at least that distance from the
+// two running sums around the chosen candidate, every such evaluation names this candidate.  Otherwise sh.safe is
+// cleared and the caller takes the exact path.  m: the number of candidates (the caller counts them).
+template <class Each, class Wt>
+__device__ __forceinline__ int walk_quick(Each each, Wt wt, float u, unsigned m, SampleShared &sh) {
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    float cs = 0.f;
+    each([&](int, float pi) { cs += wt(pi); });
+    float incl = cs;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float o = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += o;
+    }
+    __syncthreads();
+    if (lane == 63) sh.s16[wave] = incl;
+    if (t == 0) sh.first = ST;
+    __syncthreads();
+    float base = 0.f, total = 0.f;
+    for (int wv = 0; wv < ST / 64; wv++) {
+        if (wv == wave) base = total;
+        total += sh.s16[wv];
+    }
+    incl = base + incl;
+    sh.scan[t] = incl;
+    const float r = u * total;
+    if (cs > 0.f && r < incl) atomicMin(&sh.first, t);
+    __syncthreads();
+    const int c = sh.first;
+    const float tol = (6.0f * (float)m + 32.0f) * 0x1p-24f * total;
+    if (c == ST || !(tol < 0.25f * total)) { // r not clearly below the total, or too many candidates for the bound to say anything
+        if (t == 0) sh.safe = 0;
+        __syncthreads();
+        return -1;
+    }
+    if (t == c) { // walk this chunk from the running sum the chunk before it ended on
+        float cum = c ? sh.scan[c - 1] : 0.f, below = cum;
+        int res = -1;
+        each([&](int i, float pi) {
+            const float w = wt(pi);
+            if (res < 0 && w > 0.f) {
+                below = cum;
+                cum += w;
+                if (r < cum) res = i;
+            }
+        });
+        sh.result = res;
+        if (res < 0 || !(r - below > tol) || !(cum - r > tol)) sh.safe = 0;
+    }
+    __syncthreads();
+    return sh.result;
+}
+
 // top_k_sampling (sampling.zig:300-339) for k <= 1024.  Order of the reference's stable descending sort = descending
 // order of the 64-bit key (probability bits, ~index): probabilities are not negative, so their bit patterns order like
 // their values, and among equal probabilities the lower index has the larger key.  Keys are distinct, so the k largest
 // are exactly the keys >= the k-th largest, which a radix select finds 8 bits at a time without sorting the vocabulary;
 // those k are then sorted (bitonic, in LDS) and walked by one thread with the reference's sequential sums.
-template <class Each>
-__device__ __forceinline__ int top_k_walk(Each each, unsigned k, float u, SampleShared &sh) {
+// QUICK: each() yields the exps (not the probabilities), scale is a 1 / sum that need not be the reference's bits, and
+// k + 1 keys are selected.  Ordering by the exps is the reference's ordering by the probabilities (one multiplication of
+// every exp by the same factor, rounded: monotone) unless two different exps are so close that the factor can round them
+// to one value, where the index would decide instead: any two neighbours among the k + 1 must be equal or more than
+// 2^-21 apart in relative terms.  The draw must keep (6 k + 32) 2^-24 of the total away from the running sums around the
+// chosen candidate (the factor cancels in r against a running sum up to the roundings).  Both hold: the index is what
+// the exact evaluation returns; else sh.safe is cleared.
+template <bool QUICK, class Each>
+__device__ __forceinline__ int top_k_walk(Each each, unsigned k, float scale, float u, SampleShared &sh) {
     const int t = threadIdx.x, copy = t & (COPIES - 1);
-    unsigned k_rem = k, digit = 0;
+    const unsigned nsel = QUICK ? k + 1 : k; // the caller makes sure that nsel fits ST and the row
+    unsigned k_rem = nsel, digit = 0;
     // One pass of the select: count, per value of an 8-bit digit, the keys that still match everything decided so far
     // (digit_if_match gives the digit, or -1), then move on to the digit whose bucket holds the k_rem-th largest of them.
     // True when every key of that bucket is among the k: nothing below this digit needs looking at.
@@ -338,7 +415,7 @@ __device__ __forceinline__ int top_k_walk(Each each, unsigned k, float u, Sample
         }
     });
     unsigned P = 1;
-    while (P < k) P <<= 1;
+    while (P < nsel) P <<= 1;
     // Bitonic sort, descending, one key per thread: partners less than a wavefront apart trade keys through shuffles,
     // the others through LDS.
     __syncthreads();
@@ -366,14 +443,24 @@ __device__ __forceinline__ int top_k_walk(Each each, unsigned k, float u, Sample
     // of the dependent additions) and kept; every thread then tests its own candidate against r = u * total, and the
     // lowest position that passes wins.  Places past k hold probability 0: adding them changes nothing, so no step of the
     // loop is conditional.  Falls back to the last of the k.
+    if (QUICK) { // neighbours among the k + 1: equal, or clearly apart
+        if ((unsigned)t + 1 < nsel) {
+            const float a = __uint_as_float((unsigned)(sh.cand[t] >> 32)), b = __uint_as_float((unsigned)(sh.cand[t + 1] >> 32));
+            if (a != b && !(a - b > a * 0x1p-21f)) sh.safe = 0;
+        }
+    }
     if (t == 0) {
         float cum = 0.f, w[16], w_next[16];
+        auto weight = [&](unsigned j) {
+            const float x = __uint_as_float((unsigned)(sh.cand[j] >> 32));
+            return QUICK ? (j < k ? x * scale : 0.f) : x; // the probability: one multiplication (ops.zig:1598)
+        };
 #pragma unroll
-        for (int e = 0; e < 16; e++) w[e] = __uint_as_float((unsigned)(sh.cand[e] >> 32));
+        for (int e = 0; e < 16; e++) w[e] = weight(e);
         for (unsigned j0 = 0; j0 < k; j0 += 16) {
             const unsigned j1 = j0 + 16 < (unsigned)ST ? j0 + 16 : 0; // the block after this one, read while this one is added up
 #pragma unroll
-            for (int e = 0; e < 16; e++) w_next[e] = __uint_as_float((unsigned)(sh.cand[j1 + e] >> 32));
+            for (int e = 0; e < 16; e++) w_next[e] = weight(j1 + e);
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 cum += w[e];
@@ -385,10 +472,15 @@ __device__ __forceinline__ int top_k_walk(Each each, unsigned k, float u, Sample
         sh.first = (int)k - 1;
     }
     __syncthreads();
-    const float r = u * sh.scan[k - 1];
+    const float total = sh.scan[k - 1], r = u * total;
     if ((unsigned)t < k && r < sh.scan[t]) atomicMin(&sh.first, t);
     __syncthreads();
-    return (int)~(unsigned)sh.cand[sh.first];
+    const int first = sh.first;
+    if (QUICK && t == 0) {
+        const float tol = (6.0f * (float)k + 32.0f) * 0x1p-24f * total, below = first ? sh.scan[first - 1] : 0.f;
+        if (!(r - below > tol) || !(sh.scan[first] - r > tol) || !(tol < 0.25f * total)) sh.safe = 0;
+    }
+    return (int)~(unsigned)sh.cand[first];
 }
 
 // J > 0: J (even) logits per thread, probabilities kept in registers; the logits pointer is 4-byte aligned.
@@ -451,64 +543,118 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs p) {
 #pragma unroll
         for (int j = 0; j < J; j++) v[j] = e_of(v[j]);
     }
-    // the sum of the exps in the reference's sequential order (ops.zig:1585-1592; sampling.zig:139-147 for min_p)
-    const float sum = seq_prefix(
-        [&](auto f) {
-            if constexpr (J > 0) {
-#pragma unroll
-                for (int j = 0; j < J; j++) f(t * J + j, v[j]);
-            } else {
-                for (int i = lo; i < hi; i++) f(i, e_of(lg(i)));
-            }
-        },
-        sh);
-    const float inv_sum = __fdiv_rn(1.0f, sum);
-    const bool normalise = METHOD == MOON_SAMPLE_MIN_P || sum > 0.f; // ops.softmax normalises only a positive sum (ops.zig:1595; otherwise it leaves its input, the scaled logits, in place: only a not-a-number logit gets there, and the exps stand in here)
-    if constexpr (J > 0) {
-        if (normalise) {
-#pragma unroll
-            for (int j = 0; j < J; j++) v[j] = v[j] * inv_sum;
-        }
-    }
-    // f(i, probability of i) for the thread's own indices, ascending
-    auto each = [&](auto f) {
+    // v[] holds the exps from here on; a probability is one multiplication, exp * (1 / sum) (ops.zig:1598, sampling.zig:150-153)
+    float inv = 1.f;
+    bool normalise = true;
+    // f(i, exp of i) for the thread's own indices, ascending
+    auto each_exp = [&](auto f) {
         if constexpr (J > 0) {
             int first = t * J;
             asm volatile("" : "+v"(first)); // or the compiler keeps every index (and what callers derive from it) in a register of its own across the passes
 #pragma unroll
             for (int j = 0; j < J; j++) f(first + j, v[j]);
         } else {
-            for (int i = lo; i < hi; i++) {
-                const float e = e_of(lg(i));
-                f(i, normalise ? e * inv_sum : e);
-            }
+            for (int i = lo; i < hi; i++) f(i, e_of(lg(i)));
         }
     };
-
-    int token;
-    if constexpr (METHOD == MOON_SAMPLE_MULTINOMIAL) { // multinomial_sampling (sampling.zig:276-297); falls back to the last index
-        token = walk_in_index_order(each, [](float pi) { return pi; }, u, sh);
-        if (token < 0) token = n - 1;
-    } else if constexpr (METHOD == MOON_SAMPLE_MIN_P) { // min_p_sampling (sampling.zig:114-219)
-        float max_prob = 0.f;
-        each([&](int, float pi) { max_prob = fmaxf(max_prob, pi); });
-        max_prob = block_max(max_prob, sh.s16);
-        const float threshold = p.min_p * max_prob;
-        int first_valid = 0x7fffffff, first_max = 0x7fffffff;
-        each([&](int i, float pi) {
-            if (pi >= threshold) first_valid = min(first_valid, i);
-            if (pi == max_prob) first_max = min(first_max, i);
-        });
-        first_valid = block_min_int(first_valid, sh.s16i);
-        if (first_valid == 0x7fffffff) { // nothing reaches the threshold: keep the first maximum (sampling.zig:183-197)
-            token = block_min_int(first_max, sh.s16i);
-            if (token == 0x7fffffff) token = 0; // not-a-number logits
+    // f(i, probability of i)
+    auto each = [&](auto f) { each_exp([&](int i, float e) { f(i, normalise ? e * inv : e); }); };
+    // the same as a loop that stays a loop: the phases of seq_prefix run it many times, and fifty unrolled copies of their
+    // body each time cost more registers than a lane has
+    auto each_exp_rolled = [&](auto f) {
+        if constexpr (J > 0) {
+#pragma unroll 1
+            for (int j = 0; j < J; j++) f(t * J + j, v[j]);
         } else {
-            token = walk_in_index_order(each, [&](float pi) { return pi >= threshold ? pi : 0.f; }, u, sh);
-            if (token < 0) token = first_valid; // sampling.zig:217-218
+            each_exp(f);
         }
-    } else {
-        token = top_k_walk(each, (unsigned)min(p.k, n), u, sh);
+    };
+    auto each_rolled = [&](auto f) { each_exp_rolled([&](int i, float e) { f(i, normalise ? e * inv : e); }); };
+
+    // One evaluation of the method with the current 1 / sum.  quick: sums in whatever order is fast, and sh.safe is cleared
+    // unless the result provably does not depend on that (see walk_quick / top_k_walk); exact: the reference's loops, bit
+    // for bit.
+    auto run = [&](auto quick_tag) -> int {
+        constexpr bool QUICK = decltype(quick_tag)::value;
+        int token;
+        if constexpr (METHOD == MOON_SAMPLE_MULTINOMIAL) { // multinomial_sampling (sampling.zig:276-297); falls back to the last index
+            if constexpr (QUICK) {
+                token = walk_quick(each, [](float pi) { return pi; }, u, (unsigned)n, sh);
+            } else {
+                token = walk_exact(each_rolled, [](float pi) { return pi; }, u, sh);
+                if (token < 0) token = n - 1;
+            }
+        } else if constexpr (METHOD == MOON_SAMPLE_MIN_P) { // min_p_sampling (sampling.zig:114-219)
+            float max_prob = 0.f;
+            each([&](int, float pi) { max_prob = fmaxf(max_prob, pi); });
+            max_prob = block_max(max_prob, sh.s16);
+            const float threshold = p.min_p * max_prob;
+            int first_valid = 0x7fffffff, first_max = 0x7fffffff;
+            each([&](int i, float pi) {
+                if (pi >= threshold) first_valid = min(first_valid, i);
+                if (pi == max_prob) first_max = min(first_max, i);
+            });
+            first_valid = block_min_int(first_valid, sh.s16i);
+            unsigned m = 0;
+            if constexpr (QUICK) {
+                // Which indices are candidates, and which is the first maximum, must not depend on the factor either: an exp
+                // equal to the largest one or clearly below it, and clearly on one side of min_p times the largest one.
+                float e_max = 0.f;
+                each_exp([&](int, float e) { e_max = fmaxf(e_max, e); });
+                e_max = block_max(e_max, sh.s16);
+                const float edge = p.min_p * e_max;
+                int close = 0, count = 0;
+                each_exp([&](int, float e) {
+                    if (e != e_max && !(e_max - e > e_max * 0x1p-21f)) close = 1;
+                    if (fabsf(e - edge) <= edge * 0x1p-20f) close = 1;
+                    if (e > edge) count++;
+                });
+                if (close) sh.safe = 0;
+                m = (unsigned)block_sum((float)count, sh.s16); // at most 2^24 of them: the float sum is the integer
+            }
+            if (first_valid == 0x7fffffff) { // nothing reaches the threshold: keep the first maximum (sampling.zig:183-197)
+                token = block_min_int(first_max, sh.s16i);
+                if (token == 0x7fffffff) token = 0; // not-a-number logits
+            } else if constexpr (QUICK) {
+                token = walk_quick(each, [&](float pi) { return pi >= threshold ? pi : 0.f; }, u, m, sh);
+            } else {
+                token = walk_exact(each_rolled, [&](float pi) { return pi >= threshold ? pi : 0.f; }, u, sh);
+                if (token < 0) token = first_valid; // sampling.zig:217-218
+            }
+        } else {
+            const unsigned k = (unsigned)min(p.k, n);
+            if constexpr (QUICK) {
+                if (k + 1 > (unsigned)n || k + 1 > (unsigned)ST) { // no (k+1)-th key to compare the k-th with
+                    if (t == 0) sh.safe = 0;
+                    token = 0;
+                } else {
+                    token = top_k_walk<true>(each_exp, k, inv, u, sh);
+                }
+            } else {
+                token = top_k_walk<false>(each, k, 1.f, u, sh);
+            }
+        }
+        return token;
+    };
+
+    // the quick attempt: the sum of the exps as a tree
+    if (t == 0) sh.safe = 1;
+    float sum = 0.f;
+    each_exp([&](int, float e) { sum += e; });
+    sum = block_sum(sum, sh.s16); // (its barriers also publish sh.safe)
+    inv = __fdiv_rn(1.0f, sum);
+    if (!(sum > 0.f) && t == 0) sh.safe = 0; // not-a-number logits: the exact path decides
+    __syncthreads();
+    int token = run(std::true_type{});
+    __syncthreads();
+    if (!sh.safe) {
+        // the sum of the exps in the reference's sequential order (ops.zig:1585-1592; sampling.zig:139-147 for min_p)
+        sum = seq_prefix(each_exp_rolled, sh);
+        inv = __fdiv_rn(1.0f, sum);
+        // ops.softmax normalises only a positive sum (ops.zig:1595; otherwise it leaves its input, the scaled logits, in place:
+        // only a not-a-number logit gets there, and the exps stand in here); min_p always does (sampling.zig:150)
+        normalise = METHOD == MOON_SAMPLE_MIN_P || sum > 0.f;
+        token = run(std::false_type{});
     }
     if (t == 0) {
         if (p.out) p.out[0] = (uint32_t)token;
