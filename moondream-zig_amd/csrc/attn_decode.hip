@@ -33,20 +33,30 @@ __global__ void decode_attn_merge_kernel(const float *__restrict__ partial, half
 
 } // namespace
 
+int launch_decode_attention_merged(moon_ctx *ctx, const half_t *qkv, half_t *cache_k, half_t *cache_v, const float *table, float *partial,
+                                   half_t *out, uint32_t *head_count, uint32_t count_target, size_t H, size_t D, size_t rot_dim,
+                                   size_t max_seq, size_t pos, const uint32_t *pos_dev);
+
 int launch_decode_attention(moon_ctx *ctx, const half_t *qkv, half_t *cache_k, half_t *cache_v, const float *table, half_t *out,
                             size_t H, size_t D, size_t rot_dim, size_t max_seq, size_t pos, const uint32_t *pos_dev) {
     if (D != 64) return moon_fail(ctx, MOON_EINVAL_DIM, "decode attention: head_dim %zu unsupported (64 only)", D);
     if (rot_dim > D || rot_dim % 2) return moon_fail(ctx, MOON_EROT_DIM, "decode attention: bad rot_dim %zu", rot_dim);
     if (max_seq > 2048 || pos >= max_seq)
         return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "decode attention: pos %zu >= max_seq %zu (limit 2048)", pos, max_seq);
-    MOON_TRY(moon_grow(ctx, ctx->work[1], H * DEC_SPLITS * (D + 2) * sizeof(float)));
+    // One launch: the split that finishes a head last merges it (the kernel of the text session's three-kernel decode
+    // mode).  Its per-head counters sit behind the partials and count up from launch to launch.
+    const size_t partial_bytes = (H * DEC_SPLITS * (D + 2) * sizeof(float) + 255) & ~size_t(255);
+    MOON_TRY(moon_grow(ctx, ctx->work[1], partial_bytes + H * sizeof(uint32_t)));
     float *partial = (float *)ctx->work[1].ptr;
-    hipLaunchKernelGGL((decode_attn_partial_kernel<64, true>), dim3((unsigned)(H * DEC_SPLITS)), dim3(256), 0, ctx->stream, qkv, cache_k,
-                       cache_v, table, partial, (int)H, (int)rot_dim, (int)max_seq, (int)pos, pos_dev);
-    MOON_HIP(ctx, hipGetLastError());
-    hipLaunchKernelGGL(decode_attn_merge_kernel<64>, dim3((unsigned)H), dim3(64), 0, ctx->stream, partial, out);
-    MOON_HIP(ctx, hipGetLastError());
-    return MOON_OK;
+    uint32_t *head_count = reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(ctx->work[1].ptr) + partial_bytes);
+    if (ctx->attn_cnt_buf != (void *)head_count || ctx->attn_cnt_heads != H || ctx->attn_cnt_launches >= (1u << 28)) {
+        MOON_TRY(launch_fill_uniform_u32(ctx, head_count, H, 0, 0, 1)); // zeros, in stream order
+        ctx->attn_cnt_buf = head_count;
+        ctx->attn_cnt_heads = H;
+        ctx->attn_cnt_launches = 0;
+    }
+    const uint32_t target = ++ctx->attn_cnt_launches * (uint32_t)DEC_SPLITS;
+    return launch_decode_attention_merged(ctx, qkv, cache_k, cache_v, table, partial, out, head_count, target, H, D, rot_dim, max_seq, pos, pos_dev);
 }
 
 // q[H,64] already rotated, k,v[H][kv_len][64] contiguous: singleMaskedSDPA with an all-true mask.
@@ -55,6 +65,7 @@ int launch_decode_attention_plain(moon_ctx *ctx, const half_t *q, const half_t *
     if (D != 64 || kv_len == 0 || kv_len > 2048) return moon_fail(ctx, MOON_EINVAL_DIM, "plain decode attention: unsupported shape");
     MOON_TRY(moon_grow(ctx, ctx->work[1], H * DEC_SPLITS * (D + 2) * sizeof(float)));
     float *partial = (float *)ctx->work[1].ptr;
+    ctx->attn_cnt_buf = nullptr; // these partials may cover the other path's counters: it clears them before its next launch
     hipLaunchKernelGGL((decode_attn_partial_kernel<64, false>), dim3((unsigned)(H * DEC_SPLITS)), dim3(256), 0, ctx->stream, q,
                        const_cast<half_t *>(k), const_cast<half_t *>(v), (const float *)nullptr, partial, (int)H, 0, (int)kv_len,
                        (int)kv_len - 1, (const uint32_t *)nullptr);

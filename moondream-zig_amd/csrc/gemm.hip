@@ -749,77 +749,74 @@ __global__ __launch_bounds__(256) void splitk_reduce8_kernel(const float *__rest
     *reinterpret_cast<half8_t *>(C + i) = o;
 }
 
-// The split-K reduction followed by the LayerNorm of the finished rows, one wavefront per row of C (N <= 2048, N % 8 == 0):
-// the sums and the epilogue are those of splitk_reduce8_kernel (same order over the splits); the row stays in registers
-// and ops.layerNorm (ops.zig:1063-1419: f32 mean, biased variance, y = f16((x*rstd - mean*rstd)*gamma + beta)) is applied
-// to the f16 values just written to C, into ln_out.  Replaces a LayerNorm launch that would re-read C.
+// The split-K reduction followed by the LayerNorm of the finished rows, one 256-thread workgroup per row of C (N <= 2048,
+// N % 8 == 0): the sums and the epilogue are those of splitk_reduce8_kernel (same order over the splits); the row stays in
+// registers (eight columns per thread) and ops.layerNorm (ops.zig:1063-1419: f32 mean, biased variance,
+// y = f16((x*rstd - mean*rstd)*gamma + beta)) is applied to the f16 values just written to C, into ln_out.  Replaces a
+// LayerNorm launch that would re-read C.  Row sums: per wavefront, then the four wavefronts' in a fixed order.
 constexpr int LN_FUSE_MAX_N = 2048;
 template <int EPI>
 __global__ __launch_bounds__(256) void splitk_reduce_ln_kernel(const float *__restrict__ partial, const half_t *__restrict__ bias, const half_t *resid,
                                                                half_t *C, const half_t *__restrict__ gamma, const half_t *__restrict__ beta,
                                                                half_t *__restrict__ ln_out, int M, int N, int splits, float eps) {
-    const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= M) return;
+    __shared__ float s_part[2][4];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, row = blockIdx.x;
     const size_t MN = size_t(M) * N, base = size_t(row) * N;
-    half8_t v[LN_FUSE_MAX_N / 512];
+    const int n = t * 8;
+    const bool mine = n < N;
+    half8_t v = {0, 0, 0, 0, 0, 0, 0, 0}, g = v, bt = v;
     float sum = 0.0f;
+    if (mine) {
+        const size_t i = base + n;
+        float4 a = *reinterpret_cast<const float4 *>(partial + i), b = *reinterpret_cast<const float4 *>(partial + i + 4);
+        for (int k = 1; k < splits; k++) {
+            const float4 c = *reinterpret_cast<const float4 *>(partial + size_t(k) * MN + i),
+                         d = *reinterpret_cast<const float4 *>(partial + size_t(k) * MN + i + 4);
+            a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
+            b.x += d.x; b.y += d.y; b.z += d.z; b.w += d.w;
+        }
+        const float s[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        half8_t bv = {0, 0, 0, 0, 0, 0, 0, 0}, rv = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (EPI >= MOON_EPI_BIAS) bv = *reinterpret_cast<const half8_t *>(bias + n);
+        if (EPI == MOON_EPI_BIAS_RESID) rv = *reinterpret_cast<const half8_t *>(resid + i);
+        g = *reinterpret_cast<const half8_t *>(gamma + n);
+        bt = *reinterpret_cast<const half8_t *>(beta + n);
 #pragma unroll
-    for (int j = 0; j < LN_FUSE_MAX_N / 512; j++) {
-        const int n = lane * 8 + 512 * j;
-        v[j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-        if (n < N) {
-            const size_t i = base + n;
-            float4 a = *reinterpret_cast<const float4 *>(partial + i), b = *reinterpret_cast<const float4 *>(partial + i + 4);
-            for (int k = 1; k < splits; k++) {
-                const float4 c = *reinterpret_cast<const float4 *>(partial + size_t(k) * MN + i),
-                             d = *reinterpret_cast<const float4 *>(partial + size_t(k) * MN + i + 4);
-                a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
-                b.x += d.x; b.y += d.y; b.z += d.z; b.w += d.w;
-            }
-            const float s[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-            half8_t bv = {0, 0, 0, 0, 0, 0, 0, 0}, rv = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (EPI >= MOON_EPI_BIAS) bv = *reinterpret_cast<const half8_t *>(bias + n);
-            if (EPI == MOON_EPI_BIAS_RESID) rv = *reinterpret_cast<const half8_t *>(resid + i);
+        for (int e = 0; e < 8; e++) {
+            half_t o = apply_epilogue_v<EPI>(s[e], bv[e]);
+            if (EPI == MOON_EPI_BIAS_RESID) o = (half_t)((float)rv[e] + (float)o);
+            v[e] = o;
+            sum += (float)o;
+        }
+        *reinterpret_cast<half8_t *>(C + i) = v;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) s_part[0][wave] = sum;
+    __syncthreads();
+    const float mean = ((s_part[0][0] + s_part[0][1]) + (s_part[0][2] + s_part[0][3])) / (float)N;
+    float m2 = 0.0f;
+    if (mine) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                half_t o = apply_epilogue_v<EPI>(s[e], bv[e]);
-                if (EPI == MOON_EPI_BIAS_RESID) o = (half_t)((float)rv[e] + (float)o);
-                v[j][e] = o;
-                sum += (float)o;
-            }
-            *reinterpret_cast<half8_t *>(C + i) = v[j];
+        for (int e = 0; e < 8; e++) {
+            const float d = (float)v[e] - mean;
+            m2 = fmaf(d, d, m2);
         }
     }
-    const float mean = wave_sum(sum) / (float)N;
-    float m2 = 0.0f;
-#pragma unroll
-    for (int j = 0; j < LN_FUSE_MAX_N / 512; j++)
-        if (lane * 8 + 512 * j < N) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const float d = (float)v[j][e] - mean;
-                m2 = fmaf(d, d, m2);
-            }
-        }
-    const float var = wave_sum(m2) / (float)N;
+    m2 = wave_sum(m2);
+    if (lane == 0) s_part[1][wave] = m2;
+    __syncthreads();
+    const float var = ((s_part[1][0] + s_part[1][1]) + (s_part[1][2] + s_part[1][3])) / (float)N;
     const float rstd = 1.0f / sqrtf(var + eps);
-    {
+    if (mine) {
 #pragma clang fp contract(off)
         const float mean_rstd = mean * rstd; // ops.zig:1301, 1330-1333: separate multiplies and adds
+        half8_t o;
 #pragma unroll
-        for (int j = 0; j < LN_FUSE_MAX_N / 512; j++) {
-            const int n = lane * 8 + 512 * j;
-            if (n < N) {
-                const half8_t g = *reinterpret_cast<const half8_t *>(gamma + n), bt = *reinterpret_cast<const half8_t *>(beta + n);
-                half8_t o;
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const float x = (float)v[j][e] * rstd - mean_rstd;
-                    o[e] = (half_t)(x * (float)g[e] + (float)bt[e]);
-                }
-                *reinterpret_cast<half8_t *>(ln_out + base + n) = o;
-            }
+        for (int e = 0; e < 8; e++) {
+            const float x = (float)v[e] * rstd - mean_rstd;
+            o[e] = (half_t)(x * (float)g[e] + (float)bt[e]);
         }
+        *reinterpret_cast<half8_t *>(ln_out + base + n) = o;
     }
 }
 
@@ -970,7 +967,7 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
         const bool ln_ok = ln && N % 8 == 0 && N <= LN_FUSE_MAX_N && p.lds_epilogue && reinterpret_cast<uintptr_t>(ln->gamma) % 16 == 0 &&
                            reinterpret_cast<uintptr_t>(ln->beta) % 16 == 0 && reinterpret_cast<uintptr_t>(ln->out) % 16 == 0;
         if (ln_ok) {
-            hipLaunchKernelGGL(splitk_reduce_ln_kernel<EPI>, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, ctx->stream, p.partial, bias, resid, C,
+            hipLaunchKernelGGL(splitk_reduce_ln_kernel<EPI>, dim3((unsigned)M), dim3(256), 0, ctx->stream, p.partial, bias, resid, C,
                                ln->gamma, ln->beta, ln->out, M, N, splits, ln->eps);
             *ln_done = true;
         } else if (N % 8 == 0 && p.lds_epilogue)

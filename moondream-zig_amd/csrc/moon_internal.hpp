@@ -36,6 +36,11 @@ struct moon_ctx {
     GrowBuf stage[6];
     // kernel workspaces (split-K partials, attention partials, transposed B)
     GrowBuf work[3];
+    // stand-alone decode attention in one launch: per-head "splits finished" counters behind the partials in work[1]
+    // (monotonic over launches; cleared whenever the buffer or the head count changes)
+    void *attn_cnt_buf = nullptr;
+    size_t attn_cnt_heads = 0;
+    uint32_t attn_cnt_launches = 0;
     struct Resident {
         void *dptr;
         size_t n_elems;
