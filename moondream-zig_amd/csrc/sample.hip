@@ -561,10 +561,13 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs p) {
     auto each = [&](auto f) { each_exp([&](int i, float e) { f(i, normalise ? e * inv : e); }); };
     // the same as a loop that stays a loop: the phases of seq_prefix run it many times, and fifty unrolled copies of their
     // body each time cost more registers than a lane has
+    // (over a copy of the exps that is made when the exact path is entered: indexing by a loop variable puts an array in
+    // scratch memory, and the quick path's unrolled passes should keep theirs in registers)
+    float vs[J ? J : 1];
     auto each_exp_rolled = [&](auto f) {
         if constexpr (J > 0) {
 #pragma unroll 1
-            for (int j = 0; j < J; j++) f(t * J + j, v[j]);
+            for (int j = 0; j < J; j++) f(t * J + j, vs[j]);
         } else {
             each_exp(f);
         }
@@ -648,6 +651,10 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs p) {
     int token = run(std::true_type{});
     __syncthreads();
     if (!sh.safe) {
+        if constexpr (J > 0) {
+#pragma unroll
+            for (int j = 0; j < J; j++) vs[j] = v[j];
+        }
         // the sum of the exps in the reference's sequential order (ops.zig:1585-1592; sampling.zig:139-147 for min_p)
         sum = seq_prefix(each_exp_rolled, sh);
         inv = __fdiv_rn(1.0f, sum);
