@@ -8,7 +8,8 @@
 // LDS at the end.  Per tile a wave computes, with v_mfma_f32_32x32x16_f16 and f32 accumulation,
 //     S^T[key][q] = K . Q^T          (keys are the MFMA rows, so a lane holds 32 scores of ONE query and the
 //                                      row maximum / sum are in-register reductions plus one cross-half exchange)
-//     O^T[d][q]  += V^T . P^T        (P rounded to f16 for the matrix core; V is transposed while it is staged)
+//     O^T[d][q]  += V^T . P^T        (P rounded to f16 for the matrix core; V is staged row-major and transposed by
+//                                      the LDS load that feeds the matrix core)
 // The scale 1/sqrt(D) multiplies the f32 product (attention.zig:192-194, 487-489), masked scores are -inf, the
 // result is divided by the f32 row sum and rounded once to f16.
 #include "epilogue.hpp"
@@ -29,18 +30,25 @@ struct FaCfg {
     static constexpr int DT = (D + 31) / 32;      // 32-row tiles of O^T, rows >= D are zero
     static constexpr int G = D / 8;               // 16-byte granules per row
     static constexpr int KS = DK + 8;             // K tile row stride in halfs: 36 or 44 dwords, conflict-free b128 reads
-    static constexpr int VS = FA_KT + 4;          // V^T tile row stride in halfs: 34 dwords, conflict-free b64 reads
+    // The V tile stays row-major, [key][d], and is read with the transposing LDS load (ds_read_tr16_b64).  Per half-wavefront
+    // such a load touches 4 consecutive keys x 32 consecutive d: with D = 64 the rows are unpadded (32 dwords) and the 16-byte
+    // granule c of key row r sits at granule c ^ 2*(r & 3), so those 4 x 4 granules fall on distinct banks and the b128
+    // stores of two consecutive rows do too; otherwise the row stride is 48 dwords (rows 0..3 start at banks 0, 48, 32, 16).
+    static constexpr bool V_SWIZZLE = (D == 64);
+    static constexpr int VS = V_SWIZZLE ? D : 96; // V tile row stride in halfs
     static constexpr int K_HALFS = FA_KT * KS;
-    static constexpr int V_HALFS = D * VS;        // rows of O^T past D read row D-1 instead of padding (their results are dropped)
-    // the K tile and the V^T tile of a wavefront share their LDS: K is only read before the scores, V^T only after
+    static constexpr int V_HALFS = FA_KT * VS;
+    // the K tile and the V tile of a wavefront share their LDS: K is only read before the scores, V only after
     static constexpr int WAVE_HALFS = K_HALFS > V_HALFS ? K_HALFS : V_HALFS;
     static constexpr int K_LOADS = (FA_KT * G + 63) / 64;       // 16-byte loads per lane for a K tile
     static constexpr bool FA_FULL_K = (FA_KT * G) % 64 == 0;    // every lane takes part in every K load
-    static constexpr int V_TASKS = (FA_KT / 4) * G;             // (4 keys) x (8 dims) transposition tasks per tile
-    static constexpr int V_PASSES = (V_TASKS + 63) / 64;
-    static constexpr size_t MERGE_BYTES = (2 * FA_WAVES * FA_Q + FA_WAVES * DT * 32 * FA_Q) * sizeof(float);
+    // merge of the four wavefronts: O as [wave][q][SD] floats over the tiles (row stride D + 4: the 16-byte accesses of 16
+    // consecutive q fall on distinct banks), the maxima and sums [wave][q] behind them in an area of their own
+    static constexpr int SD = D + 4;
+    static constexpr size_t MERGE_BYTES = size_t(FA_WAVES) * FA_Q * SD * sizeof(float);
     static constexpr size_t TILE_BYTES = size_t(FA_WAVES) * WAVE_HALFS * sizeof(half_t);
-    static constexpr size_t LDS_BYTES = TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES;
+    static constexpr size_t ML_OFFSET = TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES;
+    static constexpr size_t LDS_BYTES = ML_OFFSET + 2 * FA_WAVES * FA_Q * sizeof(float);
 };
 
 struct FaArgs {
@@ -57,7 +65,7 @@ struct FaArgs {
 template <int D>
 struct FaTileRegs {
     u32x4 k[FaCfg<D>::K_LOADS];
-    u32x4 v[FaCfg<D>::V_PASSES][4];
+    u32x4 v[FaCfg<D>::K_LOADS];
 };
 
 // The K / V rows of a head are addressed as a buffer: a scalar descriptor of the head's rows, one 32-bit byte offset per
@@ -83,13 +91,11 @@ __device__ __forceinline__ void fa_load_v(FaTileRegs<D> &r, __amdgpu_buffer_rsrc
     using C = FaCfg<D>;
     const int tile_off = __builtin_amdgcn_readfirstlane(key0 * row_bytes);
 #pragma unroll
-    for (int ps = 0; ps < C::V_PASSES; ps++) {
-        const int task = ps * 64 + lane;
-        if (task < C::V_TASKS) {
-            const int dg = task % C::G, kq = task / C::G;
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                r.v[ps][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (4 * kq + j) * row_bytes + dg * 16, tile_off, 0));
+    for (int i = 0; i < C::K_LOADS; i++) {
+        const int g = i * 64 + lane;
+        if (C::FA_FULL_K || g < FA_KT * C::G) {
+            const int row = g / C::G, c = g % C::G;
+            r.v[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, row * row_bytes + c * 16, tile_off, 0));
         }
     }
 }
@@ -105,7 +111,7 @@ __device__ __forceinline__ void fa_store_k(const FaTileRegs<D> &r, half_t *Ks, i
             *reinterpret_cast<u32x4 *>(Ks + row * C::KS + c * 8) = r.k[i];
         }
     }
-    if (C::DK > D) { // zero padding of the contraction, columns [D, DK): one row per lane (the V^T tile overwrote it)
+    if (C::DK > D) { // zero padding of the contraction, columns [D, DK): one row per lane (the V tile overwrote it)
         static_assert(C::DK - D == 8 || C::DK == D, "one 16-byte granule of padding");
         *reinterpret_cast<u32x4 *>(Ks + lane * C::KS + D) = u32x4{0, 0, 0, 0};
     }
@@ -114,24 +120,21 @@ template <int D>
 __device__ __forceinline__ void fa_store_v(const FaTileRegs<D> &r, half_t *Vs, int lane) {
     using C = FaCfg<D>;
 #pragma unroll
-    for (int ps = 0; ps < C::V_PASSES; ps++) {
-        const int task = ps * 64 + lane;
-        if (task < C::V_TASKS) {
-            const int dg = task % C::G, kq = task / C::G;
-            half8_t rows[4];
-#pragma unroll
-            for (int j = 0; j < 4; j++) rows[j] = __builtin_bit_cast(half8_t, r.v[ps][j]);
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                half4_t t;
-                t[0] = rows[0][e];
-                t[1] = rows[1][e];
-                t[2] = rows[2][e];
-                t[3] = rows[3][e];
-                *reinterpret_cast<half4_t *>(Vs + (dg * 8 + e) * C::VS + 4 * kq) = t;
-            }
+    for (int i = 0; i < C::K_LOADS; i++) {
+        const int g = i * 64 + lane;
+        if (C::FA_FULL_K || g < FA_KT * C::G) {
+            const int row = g / C::G, c = g % C::G;
+            const int cs = C::V_SWIZZLE ? (c ^ (2 * (row & 3))) : c;
+            *reinterpret_cast<u32x4 *>(Vs + row * C::VS + cs * 8) = r.v[i];
         }
     }
+}
+// Transposing LDS load: the 16 lanes of a quarter-wavefront each name 4 consecutive halfs; lane i of the quarter receives
+// element i % 4 of the halfs named by lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12.  When lane n names key n / 4, d-columns
+// 4 * (n % 4) .. + 3 of a 4 x 16 block of row-major V, lane i ends up with column i of keys 0..3: V^T as the matrix core reads it.
+__device__ __forceinline__ half4_t fa_read_tr(const half_t *p) {
+    typedef short short4_t __attribute__((ext_vector_type(4)));
+    return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t *)(p)));
 }
 
 template <int D>
@@ -141,16 +144,46 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // (wave: a scalar)
     const int col = lane & 31, hf = lane >> 5;
     const bool causal = p.causal_pos >= 0;
+    // Workgroups are dealt to the eight accelerator dies round robin, and each die has an L2 of its own: when the count
+    // divides, die x takes the x-th eighth of the (head, query block) list, so a head's K and V are fetched into one or two
+    // L2s instead of all eight.
+    int item = (int)(blockIdx.y * gridDim.x + blockIdx.x);
+    const int n_items = (int)(gridDim.x * gridDim.y);
+    if (n_items % 8 == 0) item = (item % 8) * (n_items / 8) + item / 8;
+    const int h = item / (int)gridDim.x, bx = item % (int)gridDim.x;
     // late query blocks see the most keys: start them first
-    const int qb = causal ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
-    const int h = blockIdx.y;
+    const int qb = causal ? (int)gridDim.x - 1 - bx : bx;
     const int q0 = qb * FA_Q;
     half_t *Ks = smem + wave * C::WAVE_HALFS;
     half_t *Vs = Ks; // (shared with the K tile)
+    // where this lane points the transposing loads of O^T row tile dt (see fa_read_tr): key 4*hf + (lane % 16) / 4 of the 8 keys
+    // of a contraction half-step, d-columns 32*dt + 16*((lane / 16) % 2) + 4*(lane % 4) .. + 3.  Rows of O^T at or past D are
+    // dropped, so the lanes that would name columns past the row name its last four instead.
+    int voff[C::DT];
+    {
+        const int rq = (lane & 15) >> 2;
+#pragma unroll
+        for (int dt = 0; dt < C::DT; dt++) {
+            int colh = 32 * dt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+            if (C::V_SWIZZLE) colh = (((colh >> 3) ^ (2 * rq)) << 3) | (colh & 7);
+            else colh = min(colh, D - 4);
+            voff[dt] = (4 * hf + rq) * C::VS + colh;
+        }
+    }
     // this head's rows: (Lkv - 1) row strides and one row of D halfs
     const int row_bytes = (int)p.kv_row_stride * 2, head_bytes = (p.Lkv - 1) * row_bytes + D * 2;
     const __amdgpu_buffer_rsrc_t kh = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(p.k + size_t(h) * p.kv_head_stride), 0, head_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t vh = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(p.v + size_t(h) * p.kv_head_stride), 0, head_bytes, 0x00020000);
+
+    // keys any row of this block can see
+    long kv_end = p.Lkv;
+    if (causal && p.causal_pos + q0 + FA_Q < kv_end) kv_end = p.causal_pos + q0 + FA_Q;
+    const int n_tiles = (int)((kv_end + FA_KT - 1) / FA_KT);
+
+    // The first K tile is requested before the query rows and the first V tile after them: the scores wait for K and Q only,
+    // and the one round trip to memory that this wavefront cannot hide covers all three.
+    FaTileRegs<D> regs;
+    if (wave < n_tiles) fa_load_k<D>(regs, kh, row_bytes, wave * FA_KT, lane);
 
     // this lane's query row as the MFMA "B" operand: Q[q0 + col][16*s + 8*hf .. +7]
     half8_t qf[C::KSTEPS];
@@ -165,11 +198,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
             if (d < D) qf[s] = *reinterpret_cast<const half8_t *>(qp + d);
         }
     }
-
-    // keys any row of this block can see
-    long kv_end = p.Lkv;
-    if (causal && p.causal_pos + q0 + FA_Q < kv_end) kv_end = p.causal_pos + q0 + FA_Q;
-    const int n_tiles = (int)((kv_end + FA_KT - 1) / FA_KT);
+    if (wave < n_tiles) fa_load_v<D>(regs, vh, row_bytes, wave * FA_KT, lane);
 
     float16_t o[C::DT];
 #pragma unroll
@@ -178,13 +207,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
         for (int v = 0; v < 16; v++) o[dt][v] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f; // l_run: this lane's half of the row sum
 
-    FaTileRegs<D> regs;
-    if (wave < n_tiles) {
-        fa_load_k<D>(regs, kh, row_bytes, wave * FA_KT, lane);
-        fa_load_v<D>(regs, vh, row_bytes, wave * FA_KT, lane);
-    }
     for (int t = wave; t < n_tiles; t += FA_WAVES) {
-        asm volatile("" ::: "memory"); // the V^T tile of the previous iteration has been read: the K tile takes its place
+        asm volatile("" ::: "memory"); // the V tile of the previous iteration has been read: the K tile takes its place
         fa_store_k<D>(regs, Ks, lane);
         if (t + FA_WAVES < n_tiles) fa_load_k<D>(regs, kh, row_bytes, (t + FA_WAVES) * FA_KT, lane);
         const int key0 = t * FA_KT;
@@ -243,7 +267,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
 #pragma unroll
             for (int v = 0; v < 16; v++) o[dt][v] *= alpha;
 
-        asm volatile("" ::: "memory"); // the K tile has been read (LDS serves a wavefront in order): V^T takes its place
+        asm volatile("" ::: "memory"); // the K tile has been read (LDS serves a wavefront in order): V takes its place
         fa_store_v<D>(regs, Vs, lane);
         if (t + FA_WAVES < n_tiles) fa_load_v<D>(regs, vh, row_bytes, (t + FA_WAVES) * FA_KT, lane);
         // O^T += V^T . P^T : contraction step (kt, sp) uses the keys a lane already holds in s[kt][8*sp .. 8*sp+7],
@@ -257,9 +281,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
                 for (int e = 0; e < 8; e++) pb[e] = (half_t)s[kt][8 * sp + e];
 #pragma unroll
                 for (int dt = 0; dt < C::DT; dt++) {
-                    const half_t *vp = Vs + min(32 * dt + col, D - 1) * C::VS + 32 * kt + 16 * sp + 4 * hf;
-                    const half4_t lo = *reinterpret_cast<const half4_t *>(vp);
-                    const half4_t hi = *reinterpret_cast<const half4_t *>(vp + 8);
+                    const half_t *vp = Vs + voff[dt] + (32 * kt + 16 * sp) * C::VS;
+                    const half4_t lo = fa_read_tr(vp);
+                    const half4_t hi = fa_read_tr(vp + 8 * C::VS);
                     half8_t a;
                     a[0] = lo[0]; a[1] = lo[1]; a[2] = lo[2]; a[3] = lo[3];
                     a[4] = hi[0]; a[5] = hi[1]; a[6] = hi[2]; a[7] = hi[3];
@@ -270,15 +294,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
 
     // merge the four waves' partial results
     const float l_wave = l_run + __shfl_xor(l_run, 32);
-    __syncthreads(); // every wave is done with its staging area
-    float *sm = reinterpret_cast<float *>(smem);       // [wave][q]
-    float *sl = sm + FA_WAVES * FA_Q;                  // [wave][q]
-    float *so = sl + FA_WAVES * FA_Q;                  // [wave][d][q]
+    float *so = reinterpret_cast<float *>(smem);                                                        // [wave][q][SD]
+    float *sm = reinterpret_cast<float *>(reinterpret_cast<char *>(smem) + C::ML_OFFSET);               // [wave][q]
+    float *sl = sm + FA_WAVES * FA_Q;                                                                   // [wave][q]
     if (hf == 0) {
         sm[wave * FA_Q + col] = m_run;
         sl[wave * FA_Q + col] = l_wave;
     }
-    __syncthreads();
+    __syncthreads(); // every wave is done with its staging area, which O takes over, and has published its maximum
     float m_all = -INFINITY;
 #pragma unroll
     for (int w = 0; w < FA_WAVES; w++) m_all = fmaxf(m_all, sm[w * FA_Q + col]);
@@ -286,34 +309,43 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
 #pragma unroll
     for (int dt = 0; dt < C::DT; dt++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int d = 32 * dt + 8 * (v >> 2) + 4 * hf + (v & 3);
-            so[(wave * C::DT * 32 + d) * FA_Q + col] = o[dt][v] * f;
+        for (int j = 0; j < 4; j++) {
+            const int d = 32 * dt + 8 * j + 4 * hf; // o[dt][4*j .. 4*j+3] are rows d .. d+3 of O^T
+            if (32 * dt + 8 * j < D) {
+                float4 r;
+                r.x = o[dt][4 * j] * f;
+                r.y = o[dt][4 * j + 1] * f;
+                r.z = o[dt][4 * j + 2] * f;
+                r.w = o[dt][4 * j + 3] * f;
+                *reinterpret_cast<float4 *>(so + (wave * FA_Q + col) * C::SD + d) = r;
+            }
         }
     __syncthreads();
     {
         const int q = tid & 31;
-        float l_all = 0.0f, m2 = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < FA_WAVES; w++) m2 = fmaxf(m2, sm[w * FA_Q + q]);
+        float l_all = 0.0f;
 #pragma unroll
         for (int w = 0; w < FA_WAVES; w++) {
             const float mw = sm[w * FA_Q + q];
-            if (mw != -INFINITY) l_all += __builtin_amdgcn_exp2f(mw - m2) * sl[w * FA_Q + q];
+            if (mw != -INFINITY) l_all += __builtin_amdgcn_exp2f(mw - m_all) * sl[w * FA_Q + q];
         }
         const float inv = 1.0f / l_all;
         const int row = q0 + q;
         if (row < p.Lq) {
             for (int dg = tid >> 5; dg < C::G; dg += 8) {
+                float acc[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[e] = 0.0f;
+#pragma unroll
+                for (int w = 0; w < FA_WAVES; w++) {
+                    const float4 a = *reinterpret_cast<const float4 *>(so + (w * FA_Q + q) * C::SD + dg * 8);
+                    const float4 b = *reinterpret_cast<const float4 *>(so + (w * FA_Q + q) * C::SD + dg * 8 + 4);
+                    acc[0] += a.x; acc[1] += a.y; acc[2] += a.z; acc[3] += a.w;
+                    acc[4] += b.x; acc[5] += b.y; acc[6] += b.z; acc[7] += b.w;
+                }
                 half8_t r;
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const int d = dg * 8 + e;
-                    float acc = 0.0f;
-#pragma unroll
-                    for (int w = 0; w < FA_WAVES; w++) acc += so[(w * C::DT * 32 + d) * FA_Q + q];
-                    r[e] = (half_t)(acc * inv);
-                }
+                for (int e = 0; e < 8; e++) r[e] = (half_t)(acc[e] * inv);
                 const size_t oi = p.out_merged ? (size_t(row) * p.H + h) * D + dg * 8 : (size_t(h) * p.Lq + row) * D + dg * 8;
                 *reinterpret_cast<half8_t *>(p.out + oi) = r;
             }
