@@ -165,7 +165,7 @@ void moon_sampling_config_default(moon_sampling_config *cfg);
  * over the vocabulary are sequential f32 loops, and the candidate a draw lands on depends on their rounding: the device
  * answers from fast sums only where the answer provably does not depend on the rounding, and otherwise evaluates those
  * loops bit for bit (a few hundred microseconds; always for multinomial / min_p over thousands of near-equal
- * candidates, about one draw in 10^5 for top_k 3), so for the same exps the index is the reference's for every u.  (exp itself is the
+ * candidates, a few draws in 10^5 for top_k 3), so for the same exps the index is the reference's for every u.  (exp itself is the
  * classic two-part-reduction expf, error below one ulp, spelled out in csrc/sample.hip; a libm whose expf rounds some
  * argument differently can move a boundary by that last bit.)  top_k sorts at most 1024 candidates on the device: a
  * larger min(top_k, n) is refused with MOON_EINVAL, a deliberate limit (the reference's CLI default is 3). */

@@ -13,7 +13,7 @@
 // That evaluation costs a few hundred microseconds, so the kernel first takes its sums the fast way and keeps the answer
 // only where it provably cannot depend on how they were rounded (the draw clear of the running sums next to it by more
 // than any evaluation can move them, the candidate set clear of its thresholds); otherwise it runs the exact one.  With
-// the reference's default (top_k 3) the exact path is taken about once in 10^5 draws.
+// the reference's default (top_k 3) the exact path is taken on a few draws in 10^5.
 #pragma clang fp contract(off)
 #include "moon_internal.hpp"
 

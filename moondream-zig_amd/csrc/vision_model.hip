@@ -2,6 +2,10 @@
 // mlp (vision_model.zig:231-271, 273-343, 345-364).  The moondream.bin vision layout stores matrices [L, in, out]
 // (weights.zig:459-474); they are transposed once at load time to the k-contiguous [out, in] form the GEMM kernel
 // stages without a transposition.  Activations stay on the device for all blocks.
+// The MLP's hidden width is held padded to a multiple of 64 (4304 -> 4352: fc1 gets zero rows and zero biases, so its
+// output carries gelu(0) = 0 there; fc2 gets zero columns): every row of the fc1 activations and of the fc2 weights then
+// starts on a 128-byte line, and the 64-wide k-tiles that the fc2 product copies into LDS are whole lines instead of
+// pieces of two.  The added terms are exact zeros, so no result changes.
 #include "moon_internal.hpp"
 
 #include <vector>
@@ -9,7 +13,8 @@
 struct moon_vision_model {
     moon_ctx *ctx = nullptr;
     moon_vision_config cfg{};
-    // matrices held transposed: [L][out][in]
+    size_t fp = 0; // hidden_dim rounded up to a multiple of 64
+    // matrices held transposed: [L][out][in] (fc1: [L][fp][dim], fc2: [L][dim][fp]; fc1_b: [L][fp])
     half_t *qkv_w = nullptr, *qkv_b = nullptr, *out_w = nullptr, *out_b = nullptr, *fc1_w = nullptr, *fc1_b = nullptr,
            *fc2_w = nullptr, *fc2_b = nullptr, *n1_w = nullptr, *n1_b = nullptr, *n2_w = nullptr, *n2_b = nullptr,
            *no_w = nullptr, *no_b = nullptr;
@@ -20,7 +25,8 @@ struct moon_vision_model {
     std::vector<void *> allocs;     // weights
     std::vector<void *> act_allocs; // activations
     // front and back ends of encode_image, once attached: matrices transposed to [out][in]; the patch-embedding matrix and
-    // the patches are zero padded in k to a multiple of 16 (588 -> 592) so that the product takes the matrix-core kernel
+    // the patches are zero padded in k to a multiple of 64 (588 -> 640) so that the product takes the matrix-core kernel
+    // and its rows start on 128-byte lines
     bool io = false;
     moon_vision_io_config io_cfg{};
     size_t kp = 0; // padded patch_dim
@@ -46,7 +52,7 @@ int check_cfg(moon_ctx *ctx, const moon_vision_config *c) {
 }
 
 int alloc_weights(moon_vision_model *m) {
-    const size_t L = m->cfg.n_layers, d = m->cfg.dim, f = m->cfg.hidden_dim;
+    const size_t L = m->cfg.n_layers, d = m->cfg.dim, f = m->fp;
     MOON_TRY(dalloc(m, m->allocs, L * 3 * d * d, &m->qkv_w));
     MOON_TRY(dalloc(m, m->allocs, L * 3 * d, &m->qkv_b));
     MOON_TRY(dalloc(m, m->allocs, L * d * d, &m->out_w));
@@ -70,7 +76,7 @@ int ensure_activations(moon_vision_model *m, size_t tokens) {
     for (void *p : m->act_allocs) (void)hipFree(p);
     m->act_allocs.clear();
     m->cap_tokens = 0;
-    const size_t d = m->cfg.dim, f = m->cfg.hidden_dim;
+    const size_t d = m->cfg.dim, f = m->fp;
     MOON_TRY(dalloc(m, m->act_allocs, tokens * d, &m->x));
     MOON_TRY(dalloc(m, m->act_allocs, tokens * d, &m->ln));
     MOON_TRY(dalloc(m, m->act_allocs, tokens * 3 * d, &m->qkv));
@@ -101,7 +107,7 @@ int transpose_layers(moon_vision_model *m, const half_t *tmp, half_t *dst, size_
 
 int encode_dev(moon_vision_model *m, const half_t *x_in, size_t T, half_t *out) {
     moon_ctx *ctx = m->ctx;
-    const size_t d = m->cfg.dim, f = m->cfg.hidden_dim, H = m->cfg.n_heads, D = m->cfg.head_dim;
+    const size_t d = m->cfg.dim, f = m->fp, H = m->cfg.n_heads, D = m->cfg.head_dim; // (f: the padded hidden width)
     MOON_TRY(ensure_activations(m, T));
     MOON_HIP(ctx, hipMemcpyAsync(m->x, x_in, T * d * sizeof(half_t), hipMemcpyDeviceToDevice, ctx->stream));
     // Every LayerNorm but the first follows a product that has just finished the rows it normalises (out_proj + residual ->
@@ -173,7 +179,7 @@ int io_attach(moon_vision_model *m, const moon_vision_io_config *cfg, const moon
             if (!p) return moon_fail(ctx, MOON_EINVAL, "vision io: a weight pointer is null");
     }
     MOON_HIP(ctx, hipSetDevice(ctx->device));
-    const size_t d = m->cfg.dim, T = cfg->tokens, K = cfg->patch_dim, Kp = (K + 15) / 16 * 16, Hp = cfg->proj_hidden, O = cfg->out_dim;
+    const size_t d = m->cfg.dim, T = cfg->tokens, K = cfg->patch_dim, Kp = (K + 63) / 64 * 64, Hp = cfg->proj_hidden, O = cfg->out_dim;
     m->io_cfg = *cfg;
     m->kp = Kp;
     MOON_TRY(dalloc(m, m->allocs, d * Kp, &m->pe_w));
@@ -333,12 +339,15 @@ static int vision_create(moon_ctx *ctx, const moon_vision_config *cfg, const moo
     moon_vision_model *m = new moon_vision_model();
     m->ctx = ctx;
     m->cfg = *cfg;
-    const size_t L = cfg->n_layers, d = cfg->dim, f = cfg->hidden_dim;
+    m->fp = (cfg->hidden_dim + 63) / 64 * 64;
+    const size_t L = cfg->n_layers, d = cfg->dim, f = cfg->hidden_dim, fp = m->fp;
     int rc = alloc_weights(m);
-    half_t *tmp = nullptr; // staging for one matrix family in the file layout
+    half_t *tmp = nullptr; // staging for one matrix family in the file layout, then one padded fc2 matrix
     size_t biggest = L * 3 * d * d;
     if (L * d * f > biggest) biggest = L * d * f;
-    if (rc == MOON_OK && hipMalloc((void **)&tmp, biggest * sizeof(half_t)) != hipSuccess) rc = moon_fail(ctx, MOON_ENOMEM, "vision model: staging allocation failed");
+    if (rc == MOON_OK && hipMalloc((void **)&tmp, (biggest + fp * d) * sizeof(half_t)) != hipSuccess)
+        rc = moon_fail(ctx, MOON_ENOMEM, "vision model: staging allocation failed");
+    half_t *pad = tmp ? tmp + biggest : nullptr; // [fp][d]
     // stream numbers = 100 + declaration order of moon_vision_weights
     auto mat = [&](half_t *dst, const moon_f16 *src, size_t in, size_t outn, uint64_t stream) {
         if (rc != MOON_OK) return;
@@ -364,9 +373,37 @@ static int vision_create(moon_ctx *ctx, const moon_vision_config *cfg, const moo
     vec(m->qkv_b, w ? w->v_Wqkv_b : nullptr, L * 3 * d, 101, 0);
     mat(m->out_w, w ? w->v_out_proj_w : nullptr, d, d, 102);
     vec(m->out_b, w ? w->v_out_proj_b : nullptr, L * d, 103, 0);
-    mat(m->fc1_w, w ? w->v_fc1_w : nullptr, d, f, 104);
-    vec(m->fc1_b, w ? w->v_fc1_b : nullptr, L * f, 105, 0);
-    mat(m->fc2_w, w ? w->v_fc2_w : nullptr, f, d, 106);
+    // stage(): one matrix family into tmp in the file layout, without transposing
+    auto stage = [&](const moon_f16 *src, size_t n, uint64_t stream) {
+        if (rc != MOON_OK) return;
+        if (synthetic) rc = launch_fill_normal(ctx, tmp, n, seed, stream, std_dev);
+        else if (hipMemcpyAsync(tmp, src, n * sizeof(half_t), hipMemcpyHostToDevice, ctx->stream) != hipSuccess)
+            rc = moon_fail(ctx, MOON_EHIP, "vision model: weight upload failed");
+    };
+    auto hip_ok = [&](hipError_t e) {
+        if (rc == MOON_OK && e != hipSuccess) rc = moon_fail(ctx, MOON_EHIP, "vision model: weight setup failed: %s", hipGetErrorString(e));
+    };
+    if (fp == f) {
+        mat(m->fc1_w, w ? w->v_fc1_w : nullptr, d, f, 104);
+        vec(m->fc1_b, w ? w->v_fc1_b : nullptr, L * f, 105, 0);
+        mat(m->fc2_w, w ? w->v_fc2_w : nullptr, f, d, 106);
+    } else {
+        // fc1 [d][f] -> the first f rows of [fp][d], the rest zero; its bias the first f of fp
+        if (rc == MOON_OK) rc = launch_fill_const(ctx, m->fc1_w, L * fp * d, 0.0f);
+        stage(w ? w->v_fc1_w : nullptr, L * d * f, 104);
+        for (size_t l = 0; l < L && rc == MOON_OK; l++) rc = launch_transpose(ctx, tmp + l * d * f, m->fc1_w + l * fp * d, d, f);
+        if (rc == MOON_OK) rc = launch_fill_const(ctx, m->fc1_b, L * fp, 0.0f);
+        stage(w ? w->v_fc1_b : nullptr, L * f, 105);
+        if (rc == MOON_OK)
+            hip_ok(hipMemcpy2DAsync(m->fc1_b, fp * sizeof(half_t), tmp, f * sizeof(half_t), f * sizeof(half_t), L, hipMemcpyDeviceToDevice, ctx->stream));
+        // fc2 [f][d] -> zero rows appended to [fp][d], then transposed to [d][fp]
+        stage(w ? w->v_fc2_w : nullptr, L * f * d, 106);
+        if (rc == MOON_OK) rc = launch_fill_const(ctx, pad, fp * d, 0.0f);
+        for (size_t l = 0; l < L && rc == MOON_OK; l++) {
+            hip_ok(hipMemcpyAsync(pad, tmp + l * f * d, f * d * sizeof(half_t), hipMemcpyDeviceToDevice, ctx->stream));
+            if (rc == MOON_OK) rc = launch_transpose(ctx, pad, m->fc2_w + l * d * fp, fp, d);
+        }
+    }
     vec(m->fc2_b, w ? w->v_fc2_b : nullptr, L * d, 107, 0);
     vec(m->n1_w, w ? w->v_norm1_w : nullptr, L * d, 108, 1);
     vec(m->n1_b, w ? w->v_norm1_b : nullptr, L * d, 109, 2);
