@@ -14,6 +14,8 @@
 // result is divided by the f32 row sum and rounded once to f16.
 #include "epilogue.hpp"
 
+#include <atomic>
+
 namespace {
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -356,11 +358,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
 template <int D>
 int launch_flash(moon_ctx *ctx, const FaArgs &p) {
     using C = FaCfg<D>;
-    static bool attr_set = false; // dynamic LDS above 64 KiB needs the opt-in once per process
-    if (!attr_set) {
+    static std::atomic<bool> attr_set[64]; // the opt-in to this much dynamic LDS is per device (and per instantiation)
+    const int dev = ctx->device >= 0 && ctx->device < 64 ? ctx->device : -1;
+    if (dev < 0 || !attr_set[dev].load()) {
         MOON_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(flash_attn_kernel<D>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)C::LDS_BYTES));
-        attr_set = true;
+        if (dev >= 0) attr_set[dev].store(true);
     }
     hipLaunchKernelGGL(flash_attn_kernel<D>, dim3((unsigned)((p.Lq + FA_Q - 1) / FA_Q), (unsigned)p.H), dim3(256), C::LDS_BYTES, ctx->stream, p);
     MOON_HIP(ctx, hipGetLastError());
