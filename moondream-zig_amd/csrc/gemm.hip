@@ -754,11 +754,14 @@ __global__ __launch_bounds__(256) void splitk_reduce8_kernel(const float *__rest
 // registers (eight columns per thread) and ops.layerNorm (ops.zig:1063-1419: f32 mean, biased variance,
 // y = f16((x*rstd - mean*rstd)*gamma + beta)) is applied to the f16 values just written to C, into ln_out.  Replaces a
 // LayerNorm launch that would re-read C.  Row sums: per wavefront, then the four wavefronts' in a fixed order.
+// add (with the residual epilogue only): a second addend, C = f16(resid + f16(add + t)) with t the product after its bias:
+// the two adds of the decoder's parallel block (text_model.zig:170-171) with the product as the MLP branch.
 constexpr int LN_FUSE_MAX_N = 2048;
 template <int EPI>
 __global__ __launch_bounds__(256) void splitk_reduce_ln_kernel(const float *__restrict__ partial, const half_t *__restrict__ bias, const half_t *resid,
-                                                               half_t *C, const half_t *__restrict__ gamma, const half_t *__restrict__ beta,
-                                                               half_t *__restrict__ ln_out, int M, int N, int splits, float eps) {
+                                                               const half_t *__restrict__ add, half_t *C, const half_t *__restrict__ gamma,
+                                                               const half_t *__restrict__ beta, half_t *__restrict__ ln_out, int M, int N, int splits,
+                                                               float eps) {
     __shared__ float s_part[2][4];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, row = blockIdx.x;
     const size_t MN = size_t(M) * N, base = size_t(row) * N;
@@ -776,14 +779,16 @@ __global__ __launch_bounds__(256) void splitk_reduce_ln_kernel(const float *__re
             b.x += d.x; b.y += d.y; b.z += d.z; b.w += d.w;
         }
         const float s[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-        half8_t bv = {0, 0, 0, 0, 0, 0, 0, 0}, rv = {0, 0, 0, 0, 0, 0, 0, 0};
+        half8_t bv = {0, 0, 0, 0, 0, 0, 0, 0}, rv = {0, 0, 0, 0, 0, 0, 0, 0}, av = {0, 0, 0, 0, 0, 0, 0, 0};
         if (EPI >= MOON_EPI_BIAS) bv = *reinterpret_cast<const half8_t *>(bias + n);
         if (EPI == MOON_EPI_BIAS_RESID) rv = *reinterpret_cast<const half8_t *>(resid + i);
+        if (EPI == MOON_EPI_BIAS_RESID && add) av = *reinterpret_cast<const half8_t *>(add + i);
         g = *reinterpret_cast<const half8_t *>(gamma + n);
         bt = *reinterpret_cast<const half8_t *>(beta + n);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             half_t o = apply_epilogue_v<EPI>(s[e], bv[e]);
+            if (EPI == MOON_EPI_BIAS_RESID && add) o = (half_t)((float)av[e] + (float)o); // attn += mlp (text_model.zig:170)
             if (EPI == MOON_EPI_BIAS_RESID) o = (half_t)((float)rv[e] + (float)o);
             v[e] = o;
             sum += (float)o;
@@ -851,13 +856,17 @@ __global__ __launch_bounds__(256) void transpose_kernel(const half_t *__restrict
 }
 
 // ln: optional LayerNorm of the finished rows of C into ln->out.  *ln_done says whether it was fused (into the split-K
-// reduction); if not, the caller runs it as a launch of its own.
+// reduction); if not, the caller runs it as a launch of its own.  With ln->add set only the fused form can apply the
+// epilogue: where the product does not take it, nothing is launched and GEMM_NOT_FUSED comes back.
+constexpr int GEMM_NOT_FUSED = -1000;
 template <int EPI>
 int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias, const half_t *resid, half_t *C, int M, int N, int K,
              int b_layout, const GemmLayerNorm *ln, bool *ln_done) {
+    const bool must_fuse = ln && ln->add;
     const bool aligned = (K % 8 == 0) && (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 8 == 0) && K > 0;
     if (!aligned) {
+        if (must_fuse) return GEMM_NOT_FUSED;
         const size_t mn = size_t(M) * N;
         hipLaunchKernelGGL(gemm_generic_kernel<EPI>, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, ctx->stream, A, B, bias, resid, C,
                            M, N, K, b_layout == MOON_B_NK ? 1 : 0);
@@ -900,6 +909,7 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     static const char *force = getenv("MOON_GEMM_KERNEL");
     // More 128 x 128 tiles than CUs: the 256 x 128 kernel (MOON_GEMM_KERNEL=regs|dma keeps the 128 x 128 ones).
     if (tiles > cus && buffers_ok && K % BK == 0 && N % 8 == 0 && p.lds_epilogue && !(force && (!strcmp(force, "regs") || !strcmp(force, "dma")))) {
+        if (must_fuse) return GEMM_NOT_FUSED;
         // 192-row tiles where they fill more CUs in one round than 256-row tiles do (M = 768: four row blocks, not three)
         const int t256 = ((M + 255) / 256) * p.tiles_n, t192 = ((M + 191) / 192) * p.tiles_n;
         const bool use192 = t192 <= cus && t192 > t256 && size_t((M + 191) / 192) * 192 <= size_t((M + 255) / 256) * 256 &&
@@ -936,6 +946,10 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     splits = (K + kps - 1) / kps;
     p.splits = splits;
     p.k_per_split = kps;
+    const bool ln_ok = splits > 1 && ln && N % 8 == 0 && N <= LN_FUSE_MAX_N && p.lds_epilogue && reinterpret_cast<uintptr_t>(ln->gamma) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(ln->beta) % 16 == 0 && reinterpret_cast<uintptr_t>(ln->out) % 16 == 0 &&
+                       (!ln->add || reinterpret_cast<uintptr_t>(ln->add) % 16 == 0);
+    if (must_fuse && !ln_ok) return GEMM_NOT_FUSED;
     if (splits > 1) {
         MOON_TRY(moon_grow(ctx, ctx->work[0], size_t(splits) * M * N * sizeof(float)));
         p.partial = (float *)ctx->work[0].ptr;
@@ -964,10 +978,8 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     MOON_HIP(ctx, hipGetLastError());
     if (splits > 1) {
         const size_t mn = size_t(M) * N;
-        const bool ln_ok = ln && N % 8 == 0 && N <= LN_FUSE_MAX_N && p.lds_epilogue && reinterpret_cast<uintptr_t>(ln->gamma) % 16 == 0 &&
-                           reinterpret_cast<uintptr_t>(ln->beta) % 16 == 0 && reinterpret_cast<uintptr_t>(ln->out) % 16 == 0;
         if (ln_ok) {
-            hipLaunchKernelGGL(splitk_reduce_ln_kernel<EPI>, dim3((unsigned)M), dim3(256), 0, ctx->stream, p.partial, bias, resid, C,
+            hipLaunchKernelGGL(splitk_reduce_ln_kernel<EPI>, dim3((unsigned)M), dim3(256), 0, ctx->stream, p.partial, bias, resid, ln->add, C,
                                ln->gamma, ln->beta, ln->out, M, N, splits, ln->eps);
             *ln_done = true;
         } else if (N % 8 == 0 && p.lds_epilogue)
@@ -991,6 +1003,8 @@ int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *b
     if (b_layout != MOON_B_KN && b_layout != MOON_B_NK) return moon_fail(ctx, MOON_EINVAL, "gemm: unknown B layout %d", b_layout);
     if (ln && (!ln->gamma || !ln->beta || !ln->out)) return moon_fail(ctx, MOON_EINVAL, "gemm: the LayerNorm that follows needs gamma, beta and an output");
     if (ln && !(ln->eps > 0.0f)) return moon_fail(ctx, MOON_EEPS, "gemm: the LayerNorm that follows needs eps > 0");
+    if (ln && ln->add && (epilogue != MOON_EPI_BIAS_RESID || !ln->add_scratch))
+        return moon_fail(ctx, MOON_EINVAL, "gemm: a second addend needs the residual epilogue and a scratch buffer");
     bool ln_done = false;
     int rc;
     switch (epilogue) {
@@ -1002,6 +1016,12 @@ int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *b
         rc = run_gemm<MOON_EPI_BIAS_RESID>(ctx, A, B, bias, resid, C, (int)M, (int)N, (int)K, b_layout, ln, &ln_done);
         break;
     default: return moon_fail(ctx, MOON_EINVAL, "gemm: unknown epilogue %d", epilogue);
+    }
+    if (rc == GEMM_NOT_FUSED) { // the same arithmetic as separate launches: t = product + bias; C = f16(resid + f16(add + t)); LayerNorm
+        MOON_TRY(run_gemm<MOON_EPI_BIAS>(ctx, A, B, bias, nullptr, ln->add_scratch, (int)M, (int)N, (int)K, b_layout, nullptr, &ln_done));
+        if (C != resid) MOON_HIP(ctx, hipMemcpyAsync(C, resid, M * N * sizeof(half_t), hipMemcpyDeviceToDevice, ctx->stream));
+        MOON_TRY(launch_residual2(ctx, C, ln->add, ln->add_scratch, M * N));
+        return launch_layernorm(ctx, C, ln->gamma, ln->beta, ln->out, M, N, ln->eps);
     }
     if (rc != MOON_OK || !ln || ln_done) return rc;
     return launch_layernorm(ctx, C, ln->gamma, ln->beta, ln->out, M, N, ln->eps);

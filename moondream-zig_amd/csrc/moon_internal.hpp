@@ -76,10 +76,14 @@ int launch_gemv_nt(moon_ctx *ctx, const half_t *x, const half_t *W, const half_t
 // epilogue: a MOON_EPI_* value, or the internal MOON_EPI_BIAS_RESID (3): C = f16(resid + f16(f16(acc) + bias)), resid may be C.
 // ln: a LayerNorm of the finished rows of C into ln->out (the reference's next op on this tensor, vision_model.zig:239, 253,
 // 266): fused into the split-K reduction where the product takes that path, a launch of its own otherwise.
+// add (with epilogue 3 only): a second addend, C = f16(resid + f16(add + t)), t the product after its bias: the two adds of the
+// decoder's parallel block (text_model.zig:170-171); add_scratch: M x N halfs the library may use where that is not fused.
 struct GemmLayerNorm {
     const half_t *gamma, *beta;
     half_t *out;
     float eps;
+    const half_t *add = nullptr;
+    half_t *add_scratch = nullptr;
 };
 int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias, half_t *C,
                 size_t M, size_t N, size_t K, int b_layout, int epilogue, const half_t *resid = nullptr, const GemmLayerNorm *ln = nullptr);

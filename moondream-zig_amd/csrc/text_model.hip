@@ -326,7 +326,12 @@ struct ProfScope {
 
 // one decoder layer on n rows of m->hidden appended at position pos (text_model.zig:150-172)
 // token_dev: (decode only) the layer input is row token_dev[0] of the embedding table instead of m->hidden
-int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool pos_on_device, const uint32_t *token_dev = nullptr) {
+// chain_ln (rows of a prompt only): the LayerNorm of this layer's input is already in m->ln_in unless this is the first layer,
+// and unless this is the last layer the fc2 product finishes the block itself: its split-K reduction adds the bias, the
+// attention branch and the residual and normalises the new rows with the next layer's LayerNorm (one launch instead of four;
+// launch_gemm falls back to the separate launches, same arithmetic, where the product takes no split K).
+int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool pos_on_device, const uint32_t *token_dev = nullptr,
+                  bool chain_ln = false) {
     moon_ctx *ctx = m->ctx;
     const Sizes z = sizes(m->cfg);
     const half_t *ln_w = m->ln_w + layer * z.d, *ln_b = m->ln_b + layer * z.d;
@@ -380,7 +385,7 @@ int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool p
         return launch_decode_out_fc2(ctx, m->attn, m->fc1, out_w, out_b, fc2_w, fc2_b, m->hidden, x, token_dev, z.d, z.ffn);
     }
     if (token_dev) MOON_TRY(launch_embed(ctx, m->wte, token_dev, m->hidden, 1, z.d));
-    MOON_TRY(launch_layernorm(ctx, m->hidden, ln_w, ln_b, m->ln_in, n, z.d, m->cfg.ln_eps));
+    if (!chain_ln || layer == 0) MOON_TRY(launch_layernorm(ctx, m->hidden, ln_w, ln_b, m->ln_in, n, z.d, m->cfg.ln_eps));
     if (n == 1) {
         MOON_TRY(launch_gemv_nt(ctx, m->ln_in, qkv_w, qkv_b, m->qkv, 3 * z.d, z.d, MOON_EPI_BIAS));
         MOON_TRY(launch_decode_attention(ctx, m->qkv, ck, cv, m->freqs, m->attn, z.H, z.D, m->cfg.rot_dim, z.S, pos,
@@ -394,6 +399,12 @@ int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool p
         MOON_TRY(launch_sdpa(ctx, m->q_rot, ck, cv, m->attn, z.H, n, pos + n, z.D, z.S * z.D, (long)pos, nullptr, 0, true));
         MOON_TRY(launch_gemm(ctx, m->attn, out_w, out_b, m->attn_proj, n, z.d, z.d, MOON_B_NK, MOON_EPI_BIAS));
         MOON_TRY(launch_gemm(ctx, m->ln_in, fc1_w, fc1_b, m->fc1, n, z.ffn, z.d, MOON_B_NK, MOON_EPI_BIAS_GELU));
+        if (chain_ln && layer + 1 < z.L) {
+            GemmLayerNorm next{m->ln_w + (layer + 1) * z.d, m->ln_b + (layer + 1) * z.d, m->ln_in, m->cfg.ln_eps};
+            next.add = m->attn_proj;
+            next.add_scratch = m->mlp;
+            return launch_gemm(ctx, m->fc1, fc2_w, fc2_b, m->hidden, n, z.d, z.ffn, MOON_B_NK, 3 /* bias, then += into hidden */, m->hidden, &next);
+        }
         MOON_TRY(launch_gemm(ctx, m->fc1, fc2_w, fc2_b, m->mlp, n, z.d, z.ffn, MOON_B_NK, MOON_EPI_BIAS));
     }
     return launch_residual2(ctx, m->hidden, m->attn_proj, m->mlp, n * z.d);
@@ -562,7 +573,7 @@ extern "C" int moon_text_forward(moon_text_model *m, const uint32_t *ids, size_t
     MOON_HIP(ctx, hipSetDevice(ctx->device));
     MOON_HIP(ctx, hipMemcpyAsync(m->ids_dev, ids, n_ids * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
     MOON_TRY(launch_embed(ctx, m->wte, m->ids_dev, m->hidden, n_ids, m->cfg.dim));
-    for (size_t l = 0; l < m->cfg.n_layers; l++) MOON_TRY(layer_forward(m, l, n_ids, m->cur_len, false));
+    for (size_t l = 0; l < m->cfg.n_layers; l++) MOON_TRY(layer_forward(m, l, n_ids, m->cur_len, false, nullptr, n_ids > 1));
     m->cur_len += n_ids;
     m->last_n = n_ids;
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->state_dev, (uint32_t)m->cur_len, 0u);
