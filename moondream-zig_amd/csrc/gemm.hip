@@ -759,7 +759,8 @@ __global__ __launch_bounds__(256) void splitk_reduce8_kernel(const float *__rest
 constexpr int LN_FUSE_MAX_N = 2048;
 template <int EPI>
 __global__ __launch_bounds__(256) void splitk_reduce_ln_kernel(const float *__restrict__ partial, const half_t *__restrict__ bias, const half_t *resid,
-                                                               const half_t *__restrict__ add, half_t *C, const half_t *__restrict__ gamma,
+                                                               const half_t *__restrict__ add, const float *__restrict__ add_partial, int add_splits,
+                                                               const half_t *__restrict__ add_bias, half_t *C, const half_t *__restrict__ gamma,
                                                                const half_t *__restrict__ beta, half_t *__restrict__ ln_out, int M, int N, int splits,
                                                                float eps) {
     __shared__ float s_part[2][4];
@@ -782,13 +783,25 @@ __global__ __launch_bounds__(256) void splitk_reduce_ln_kernel(const float *__re
         half8_t bv = {0, 0, 0, 0, 0, 0, 0, 0}, rv = {0, 0, 0, 0, 0, 0, 0, 0}, av = {0, 0, 0, 0, 0, 0, 0, 0};
         if (EPI >= MOON_EPI_BIAS) bv = *reinterpret_cast<const half8_t *>(bias + n);
         if (EPI == MOON_EPI_BIAS_RESID) rv = *reinterpret_cast<const half8_t *>(resid + i);
-        if (EPI == MOON_EPI_BIAS_RESID && add) av = *reinterpret_cast<const half8_t *>(add + i);
+        if (EPI == MOON_EPI_BIAS_RESID && add_partial) { // the other product's reduction and bias, as splitk_reduce8_kernel<MOON_EPI_BIAS> does them
+            float4 pa = *reinterpret_cast<const float4 *>(add_partial + i), pb = *reinterpret_cast<const float4 *>(add_partial + i + 4);
+            for (int k = 1; k < add_splits; k++) {
+                const float4 c = *reinterpret_cast<const float4 *>(add_partial + size_t(k) * MN + i),
+                             d = *reinterpret_cast<const float4 *>(add_partial + size_t(k) * MN + i + 4);
+                pa.x += c.x; pa.y += c.y; pa.z += c.z; pa.w += c.w;
+                pb.x += d.x; pb.y += d.y; pb.z += d.z; pb.w += d.w;
+            }
+            const float sa[8] = {pa.x, pa.y, pa.z, pa.w, pb.x, pb.y, pb.z, pb.w};
+            const half8_t abv = *reinterpret_cast<const half8_t *>(add_bias + n);
+#pragma unroll
+            for (int e = 0; e < 8; e++) av[e] = apply_epilogue_v<MOON_EPI_BIAS>(sa[e], abv[e]);
+        } else if (EPI == MOON_EPI_BIAS_RESID && add) av = *reinterpret_cast<const half8_t *>(add + i);
         g = *reinterpret_cast<const half8_t *>(gamma + n);
         bt = *reinterpret_cast<const half8_t *>(beta + n);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             half_t o = apply_epilogue_v<EPI>(s[e], bv[e]);
-            if (EPI == MOON_EPI_BIAS_RESID && add) o = (half_t)((float)av[e] + (float)o); // attn += mlp (text_model.zig:170)
+            if (EPI == MOON_EPI_BIAS_RESID && (add || add_partial)) o = (half_t)((float)av[e] + (float)o); // attn += mlp (text_model.zig:170)
             if (EPI == MOON_EPI_BIAS_RESID) o = (half_t)((float)rv[e] + (float)o);
             v[e] = o;
             sum += (float)o;
@@ -861,8 +874,10 @@ __global__ __launch_bounds__(256) void transpose_kernel(const half_t *__restrict
 constexpr int GEMM_NOT_FUSED = -1000;
 template <int EPI>
 int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias, const half_t *resid, half_t *C, int M, int N, int K,
-             int b_layout, const GemmLayerNorm *ln, bool *ln_done) {
-    const bool must_fuse = ln && ln->add;
+             int b_layout, const GemmLayerNorm *ln, bool *ln_done, const float **keep_partial = nullptr, int *keep_splits = nullptr) {
+    // keep_partial: run the split-K product only and leave its partials in work[3] (see launch_gemm_partials); like a second
+    // addend this is all or nothing
+    const bool must_fuse = (ln && ln->add) || keep_partial;
     const bool aligned = (K % 8 == 0) && (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(C) % 8 == 0) && K > 0;
     if (!aligned) {
@@ -949,10 +964,13 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     const bool ln_ok = splits > 1 && ln && N % 8 == 0 && N <= LN_FUSE_MAX_N && p.lds_epilogue && reinterpret_cast<uintptr_t>(ln->gamma) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(ln->beta) % 16 == 0 && reinterpret_cast<uintptr_t>(ln->out) % 16 == 0 &&
                        (!ln->add || reinterpret_cast<uintptr_t>(ln->add) % 16 == 0);
-    if (must_fuse && !ln_ok) return GEMM_NOT_FUSED;
+    if (keep_partial) {
+        if (splits <= 1 || N % 8 || !p.lds_epilogue) return GEMM_NOT_FUSED;
+    } else if (must_fuse && !ln_ok) return GEMM_NOT_FUSED;
     if (splits > 1) {
-        MOON_TRY(moon_grow(ctx, ctx->work[0], size_t(splits) * M * N * sizeof(float)));
-        p.partial = (float *)ctx->work[0].ptr;
+        GrowBuf &ws = ctx->work[keep_partial ? 3 : 0];
+        MOON_TRY(moon_grow(ctx, ws, size_t(splits) * M * N * sizeof(float)));
+        p.partial = (float *)ws.ptr;
     }
     const int total = tiles * splits;
     const int grid = ((total + 7) / 8) * 8;
@@ -976,11 +994,16 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
         hipLaunchKernelGGL(gemm_nt_mfma_kernel<EPI>, dim3(grid), dim3(256), 0, ctx->stream, p);
     }
     MOON_HIP(ctx, hipGetLastError());
+    if (keep_partial) {
+        *keep_partial = p.partial;
+        *keep_splits = splits;
+        return MOON_OK;
+    }
     if (splits > 1) {
         const size_t mn = size_t(M) * N;
         if (ln_ok) {
-            hipLaunchKernelGGL(splitk_reduce_ln_kernel<EPI>, dim3((unsigned)M), dim3(256), 0, ctx->stream, p.partial, bias, resid, ln->add, C,
-                               ln->gamma, ln->beta, ln->out, M, N, splits, ln->eps);
+            hipLaunchKernelGGL(splitk_reduce_ln_kernel<EPI>, dim3((unsigned)M), dim3(256), 0, ctx->stream, p.partial, bias, resid, ln->add,
+                               ln->add_partial, ln->add_splits, ln->add_bias, C, ln->gamma, ln->beta, ln->out, M, N, splits, ln->eps);
             *ln_done = true;
         } else if (N % 8 == 0 && p.lds_epilogue)
             hipLaunchKernelGGL(splitk_reduce8_kernel<EPI>, dim3((unsigned)((mn / 8 + 255) / 256)), dim3(256), 0, ctx->stream, p.partial, bias,
@@ -1005,6 +1028,8 @@ int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *b
     if (ln && !(ln->eps > 0.0f)) return moon_fail(ctx, MOON_EEPS, "gemm: the LayerNorm that follows needs eps > 0");
     if (ln && ln->add && (epilogue != MOON_EPI_BIAS_RESID || !ln->add_scratch))
         return moon_fail(ctx, MOON_EINVAL, "gemm: a second addend needs the residual epilogue and a scratch buffer");
+    if (ln && ln->add_partial && (!ln->add || !ln->add_bias || ln->add_splits < 2 || N % 8 || reinterpret_cast<uintptr_t>(ln->add_bias) % 16))
+        return moon_fail(ctx, MOON_EINVAL, "gemm: partials as the second addend need their bias, their split count and a destination");
     bool ln_done = false;
     int rc;
     switch (epilogue) {
@@ -1018,6 +1043,12 @@ int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *b
     default: return moon_fail(ctx, MOON_EINVAL, "gemm: unknown epilogue %d", epilogue);
     }
     if (rc == GEMM_NOT_FUSED) { // the same arithmetic as separate launches: t = product + bias; C = f16(resid + f16(add + t)); LayerNorm
+        if (ln->add_partial) {
+            const size_t mn = M * N;
+            hipLaunchKernelGGL(splitk_reduce8_kernel<MOON_EPI_BIAS>, dim3((unsigned)((mn / 8 + 255) / 256)), dim3(256), 0, ctx->stream, ln->add_partial,
+                               ln->add_bias, nullptr, const_cast<half_t *>(ln->add), mn, (int)N, ln->add_splits);
+            MOON_HIP(ctx, hipGetLastError());
+        }
         MOON_TRY(run_gemm<MOON_EPI_BIAS>(ctx, A, B, bias, nullptr, ln->add_scratch, (int)M, (int)N, (int)K, b_layout, nullptr, &ln_done));
         if (C != resid) MOON_HIP(ctx, hipMemcpyAsync(C, resid, M * N * sizeof(half_t), hipMemcpyDeviceToDevice, ctx->stream));
         MOON_TRY(launch_residual2(ctx, C, ln->add, ln->add_scratch, M * N));
@@ -1025,6 +1056,24 @@ int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *b
     }
     if (rc != MOON_OK || !ln || ln_done) return rc;
     return launch_layernorm(ctx, C, ln->gamma, ln->beta, ln->out, M, N, ln->eps);
+}
+
+int launch_gemm_partials(moon_ctx *ctx, const half_t *A, const half_t *B, size_t M, size_t N, size_t K, int b_layout, const float **partial,
+                         int *splits) {
+    *partial = nullptr;
+    *splits = 0;
+    if (M == 0 || N == 0 || M > 0x3fffffff || N > 0x3fffffff || K > 0x3fffffff) return MOON_OK;
+    if (b_layout != MOON_B_KN && b_layout != MOON_B_NK) return moon_fail(ctx, MOON_EINVAL, "gemm: unknown B layout %d", b_layout);
+    bool ln_done = false;
+    // (C only enters the alignment checks of the shared code: the workspace itself is what gets written)
+    const int rc = run_gemm<MOON_EPI_NONE>(ctx, A, B, nullptr, nullptr, reinterpret_cast<half_t *>(ctx->work[3].ptr), (int)M, (int)N, (int)K, b_layout,
+                                           nullptr, &ln_done, partial, splits);
+    if (rc == GEMM_NOT_FUSED) {
+        *partial = nullptr;
+        *splits = 0;
+        return MOON_OK;
+    }
+    return rc;
 }
 
 // dst[cols, rows] = src[rows, cols]^T

@@ -35,7 +35,7 @@ struct moon_ctx {
     // staging for host-pointer ops: a, b, c, bias/aux, mask
     GrowBuf stage[6];
     // kernel workspaces (split-K partials, attention partials, transposed B)
-    GrowBuf work[3];
+    GrowBuf work[4]; // 0: split-K partials, 1: decode-attention partials, 2: transposed operands, 3: split-K partials kept for a later launch
     // stand-alone decode attention in one launch: per-head "splits finished" counters behind the partials in work[1]
     // (monotonic over launches; cleared whenever the buffer or the head count changes)
     void *attn_cnt_buf = nullptr;
@@ -84,7 +84,18 @@ struct GemmLayerNorm {
     float eps;
     const half_t *add = nullptr;
     half_t *add_scratch = nullptr;
+    // the second addend as the split-K partials of an earlier product that launch_gemm_partials left behind, with that product's
+    // bias: add = f16(f16(sum of the partials) + add_bias) is then formed on the fly (add must still name M x N halfs, which
+    // receive it where the epilogue is not fused)
+    const float *add_partial = nullptr;
+    int add_splits = 0;
+    const half_t *add_bias = nullptr;
 };
+// The split-K product of launch_gemm without its reduction: the f32 partials [splits][M][N] stay in a workspace of the context
+// (valid until the next call of this function) for a later launch_gemm to fold in through GemmLayerNorm::add_partial.
+// *splits = 0 (nothing launched) where the shape does not take the split-K path.
+int launch_gemm_partials(moon_ctx *ctx, const half_t *A, const half_t *B, size_t M, size_t N, size_t K, int b_layout, const float **partial,
+                         int *splits);
 int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias, half_t *C,
                 size_t M, size_t N, size_t K, int b_layout, int epilogue, const half_t *resid = nullptr, const GemmLayerNorm *ln = nullptr);
 

@@ -328,8 +328,9 @@ struct ProfScope {
 // token_dev: (decode only) the layer input is row token_dev[0] of the embedding table instead of m->hidden
 // chain_ln (rows of a prompt only): the LayerNorm of this layer's input is already in m->ln_in unless this is the first layer,
 // and unless this is the last layer the fc2 product finishes the block itself: its split-K reduction adds the bias, the
-// attention branch and the residual and normalises the new rows with the next layer's LayerNorm (one launch instead of four;
-// launch_gemm falls back to the separate launches, same arithmetic, where the product takes no split K).
+// attention branch (reducing out_proj's split K on the way) and the residual and normalises the new rows with the next
+// layer's LayerNorm (one launch instead of five; launch_gemm falls back to the separate launches, same arithmetic, where a
+// product takes no split K).
 int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool pos_on_device, const uint32_t *token_dev = nullptr,
                   bool chain_ln = false) {
     moon_ctx *ctx = m->ctx;
@@ -397,12 +398,22 @@ int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool p
         MOON_TRY(launch_gemm(ctx, m->ln_in, qkv_w, qkv_b, m->qkv, n, 3 * z.d, z.d, MOON_B_NK, MOON_EPI_BIAS));
         MOON_TRY(launch_qkv_rope_cache(ctx, m->qkv, m->q_rot, ck, cv, m->freqs, n, z.H, z.D, m->cfg.rot_dim, z.S, pos));
         MOON_TRY(launch_sdpa(ctx, m->q_rot, ck, cv, m->attn, z.H, n, pos + n, z.D, z.S * z.D, (long)pos, nullptr, 0, true));
-        MOON_TRY(launch_gemm(ctx, m->attn, out_w, out_b, m->attn_proj, n, z.d, z.d, MOON_B_NK, MOON_EPI_BIAS));
+        const bool finish_in_fc2 = chain_ln && layer + 1 < z.L;
+        // where fc2 finishes the block, out_proj leaves its split-K partials for that launch to reduce as well
+        const float *out_partial = nullptr;
+        int out_splits = 0;
+        if (finish_in_fc2) MOON_TRY(launch_gemm_partials(ctx, m->attn, out_w, n, z.d, z.d, MOON_B_NK, &out_partial, &out_splits));
+        if (!out_splits) MOON_TRY(launch_gemm(ctx, m->attn, out_w, out_b, m->attn_proj, n, z.d, z.d, MOON_B_NK, MOON_EPI_BIAS));
         MOON_TRY(launch_gemm(ctx, m->ln_in, fc1_w, fc1_b, m->fc1, n, z.ffn, z.d, MOON_B_NK, MOON_EPI_BIAS_GELU));
-        if (chain_ln && layer + 1 < z.L) {
+        if (finish_in_fc2) {
             GemmLayerNorm next{m->ln_w + (layer + 1) * z.d, m->ln_b + (layer + 1) * z.d, m->ln_in, m->cfg.ln_eps};
             next.add = m->attn_proj;
             next.add_scratch = m->mlp;
+            if (out_splits) {
+                next.add_partial = out_partial;
+                next.add_splits = out_splits;
+                next.add_bias = out_b;
+            }
             return launch_gemm(ctx, m->fc1, fc2_w, fc2_b, m->hidden, n, z.d, z.ffn, MOON_B_NK, 3 /* bias, then += into hidden */, m->hidden, &next);
         }
         MOON_TRY(launch_gemm(ctx, m->fc1, fc2_w, fc2_b, m->mlp, n, z.d, z.ffn, MOON_B_NK, MOON_EPI_BIAS));
