@@ -136,3 +136,27 @@ def test_matrix_core_attention_peaked_softmax(moon, O, ctx):
     out = moon.attention.multi_maskless_sdpa(H, D, q, k, v, ctx=ctx)
     assert np.isfinite(out.astype(np.float32)).all()
     assert O.rel_frobenius(out, O.sdpa_multi(q, k, v, None)) <= TOL
+
+
+def test_matrix_core_attention_over_seeded_random_shapes(moon, O, ctx):
+    """The matrix-core kernel over shapes no other test names: head counts 1..32 (multiples of 8 take the die-wise work
+    mapping), 16..300 rows, head_dim 64 (causal with a past, and maskless) and 72, keys not a multiple of the 64-key tile."""
+    rng = np.random.default_rng(1)
+    worst = 0.0
+    for it in range(48):
+        D = 72 if it % 2 else 64
+        H = int(rng.integers(1, 9)) if it % 5 else 8 * int(rng.integers(1, 5))
+        S = int(rng.integers(16, 300))
+        q = O.fill_normal_f16((H, S, D), it, 0, 1.0)
+        if D == 64 and it % 3 == 0:
+            pos = int(rng.integers(0, 200))
+            k, v = O.fill_normal_f16((H, pos + S, D), it, 1, 1.0), O.fill_normal_f16((H, pos + S, D), it, 2, 1.0)
+            mask = moon.attention.create_attention_mask(pos, S)
+            out, want = moon.attention.multi_masked_sdpa(q, k, v, mask, H, D, ctx=ctx), O.sdpa_multi(q, k, v, mask)
+        else:
+            k, v = O.fill_normal_f16((H, S, D), it, 1, 1.0), O.fill_normal_f16((H, S, D), it, 2, 1.0)
+            out, want = moon.attention.multi_maskless_sdpa(H, D, q, k, v, ctx=ctx), O.sdpa_multi(q, k, v, None)
+        err = O.rel_frobenius(out, want)
+        assert err <= TOL, (it, D, H, S, err)
+        worst = max(worst, err)
+    print(f"\nworst rel-Frobenius over 48 shapes: {worst:.2e}")
