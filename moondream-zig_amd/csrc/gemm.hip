@@ -275,14 +275,14 @@ __device__ __forceinline__ void gemm_park_tile(const float16_t (&acc)[2][2], int
                 *reinterpret_cast<half4_t *>(scratch + (wm * 64 + mi * 32 + frag_row) * TILE_PITCH + wn * 64 + ni * 32 + 8 * q + 4 * frag_g) = o;
             }
 }
-template <int EPI>
+template <int EPI, int ROWS = 128> // ROWS: rows of the parked tile (32 per pass of the 512 threads)
 __device__ __forceinline__ void gemm_tile_out(const GemmArgs &p, int m0, int n0, int t, const half_t *scratch) {
     const int nl = (t & 15) * 8, n = n0 + nl;
     if (n >= p.N) return;
     half8_t bias = {0, 0, 0, 0, 0, 0, 0, 0};
     if (EPI >= MOON_EPI_BIAS) bias = *reinterpret_cast<const half8_t *>(p.bias + n);
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
+    for (int r = 0; r < ROWS / 32; r++) {
         const int ml = r * 32 + (t >> 4), m = m0 + ml;
         if (m >= p.M) continue;
         const half8_t v = *reinterpret_cast<const half8_t *>(scratch + ml * TILE_PITCH + nl);
@@ -533,6 +533,8 @@ template <int EPI, int MI>
 __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p) {
     static_assert(MI == 3 || MI == 4, "192- or 256-row tiles");
     constexpr int BM2 = Dma2<MI>::BM2, STAGE2_HALFS = Dma2<MI>::STAGE2_HALFS, A_LOADS = Dma2<MI>::A_LOADS;
+    constexpr bool SHARED_EPILOGUE = EPI == MOON_EPI_BIAS_GELU; // all eight wavefronts finish the tile
+    static_assert(size_t(BM2) * TILE_PITCH <= size_t(DMA2_STAGES) * STAGE2_HALFS, "the parked tile fits the staging area");
     extern __shared__ __attribute__((aligned(16))) half_t lds2[]; // [stage][act: 256 rows | weight: 128 rows][64 halfs]
 
     const int total = p.tiles_m * p.tiles_n;
@@ -594,6 +596,11 @@ __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p) {
                 wait_tile(kt + 1);
                 lds_barrier(); // publishes tile kt+1
             }
+        }
+        if constexpr (SHARED_EPILOGUE) { // the loaders take their half of the epilogue (see the multipliers' end)
+            lds_barrier();               // the multipliers have read the last k-tile
+            lds_barrier();               // ... and parked the tile
+            gemm_tile_out<EPI, BM2>(p, m0, n0, t, lds2);
         }
         return;
     }
@@ -678,6 +685,26 @@ __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p) {
     first_three(n_ktiles - 1);
     wait_all(fa[1], fw[1]);
     multiply(fa[1], fw[1]);
+    if constexpr (SHARED_EPILOGUE) {
+        // With GELU the epilogue is VALU work and the loaders have nothing left to do: the multipliers park the whole tile in
+        // LDS as f16 ([m][n], pitch 136 halfs, from the start of the staging area, which is free once every multiplier has
+        // read the last k-tile), and all eight wavefronts finish it, eight consecutive n of BM2 / 32 rows per thread.
+        lds_barrier();
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+            for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    half4_t o;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[e] = (half_t)acc[ni][mi][4 * q + e];
+                    *reinterpret_cast<half4_t *>(lds2 + (wm * 32 * MI + mi * 32 + frag_row) * TILE_PITCH + wn * 64 + ni * 32 + 8 * q + 4 * frag_g) = o;
+                }
+        lds_barrier();
+        gemm_tile_out<EPI, BM2>(p, m0, n0, t, lds2);
+        return;
+    }
     // the stage after the last k-tile's is free (every copy into it has landed and been read): 64 x 68 halfs per wavefront
     half_t *scratch = lds2 + size_t(n_ktiles % DMA2_STAGES) * STAGE2_HALFS + size_t(role_wave) * 64 * EPI_PITCH;
     { // the first 64 rows of the sub-tile
