@@ -17,14 +17,14 @@ __device__ __forceinline__ float gelu_f32(float v) {
     // constants are the f16-rounded values the reference uses (ops.zig:1641-1642)
     const float c = 0.7978515625f, alpha = 0.044708251953125f;
     const float cube = v * v * v;
-    const float inner = c * (v + alpha * cube);
-    // tanh(x) = 1 - 2 / (exp(2x) + 1) on the hardware's exp2 and reciprocal (each within an ulp; the limits +-1 come out
-    // exactly).  Only 1 + t enters the result, so the absolute error of t (~2e-7) is what counts: three orders below
-    // the f16 spacing of the result.  The library tanhf costs ~45 instructions per element, which made the GELU epilogue
-    // of the vision fc1 GEMM 6 us of its 22.
-    const float e = __builtin_amdgcn_exp2f(inner * 2.8853900817779268f); // exp(2 * inner)
-    const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
-    return f32_round(0.5f * v * (1.0f + t));
+    // 0.5 v (1 + tanh(u)) = v / (1 + exp(-2u)), u = c (v + alpha v^3): one exp2 and one reciprocal of the hardware (each
+    // within an ulp), no cancellation for negative v, the limits v and -0 come out exactly.  The error against the
+    // reference's f32 evaluation with a library tanh is a few f32 ulps of the result: three orders below the f16 spacing.
+    // The library tanhf costs ~45 instructions per element, which made the GELU epilogue of the vision fc1 GEMM 6 us of
+    // its 22; this form is 7 plain instructions and the two transcendental ones.
+    const float z = (c * 2.8853900817779268f) * (v + alpha * cube); // 2u / ln 2
+    const float e = __builtin_amdgcn_exp2f(-z);
+    return f32_round(v * __builtin_amdgcn_rcpf(1.0f + e));
 }
 
 // epilogue with the bias value already in hand
