@@ -264,10 +264,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
                 psum += e;
             }
         l_run = l_run * alpha + psum;
+        // (rows of O^T at or past D are never read: in the last row tile only the registers of rows below D are rescaled;
+        // the others hold whatever accumulates, each on its own)
 #pragma unroll
         for (int dt = 0; dt < C::DT; dt++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) o[dt][v] *= alpha;
+            for (int v = 0; v < 16; v++)
+                if (32 * dt + 8 * (v >> 2) < D) o[dt][v] *= alpha;
 
         asm volatile("" ::: "memory"); // the K tile has been read (LDS serves a wavefront in order): V takes its place
         fa_store_v<D>(regs, Vs, lane);
