@@ -83,6 +83,11 @@ int moon_ctx_create(int device, moon_ctx **out);
 void moon_ctx_destroy(moon_ctx *ctx);
 /* Text of the last error on this ctx (or of the last failed moon_ctx_create when ctx is NULL). */
 const char *moon_last_error(const moon_ctx *ctx);
+/* Measurement and test knob without a counterpart in the reference: names the matrix-product kernel that moon_hgemm,
+ * moon_hgemm_trans, moon_linear and the sessions of this context take wherever the shape allows it ("regs", "dma",
+ * "dma256", "w114", "w212", "w221"; "" or NULL: chosen by shape, the default).  Every kernel computes the same product to
+ * the same rounding points; only the time changes.  The context starts with the value of MOON_GEMM_KERNEL. */
+int moon_set_gemm_kernel(moon_ctx *ctx, const char *name);
 int moon_sync(moon_ctx *ctx);
 /* Releases workspaces. Replaces attention.cleanupThreadPool() (attention.zig:814-818): the
  * reference frees its persistent worker pool there; here it drops cached device buffers. */
@@ -399,7 +404,7 @@ int moon_bin_vision_io_weights(const moon_bin *bin, const moon_vision_config *cf
  *   MOON_LAYER_QKV_WGS=n           decode mode 0: workgroups that take qkv rows (default: the attention and output workgroups)
  *   MOON_LAYER_FC1_OUT_ROWS=n      decode mode 0: fc1 rows per output wavefront (default: half an fc1-only wavefront's share)
  *   MOON_LAYER_FC1_GROUP=1|2       decode mode 0: fc1 rows a wavefront requests together (default 1)
- *   MOON_GEMM_KERNEL=regs|dma|dma256  forces one of the MFMA product kernels where the shape allows it (default: by shape)
+ *   MOON_GEMM_KERNEL=regs|dma|dma256|w114|w212|w221  forces one of the MFMA product kernels where the shape allows it (default: by shape)
  *   MOON_GEMM_EPILOGUE=direct      the product kernels store their tile without the pass through LDS (default: through LDS)
  * Every setting gives the same results (bit for bit, MOON_STREAM_DEBUG aside); only the time changes. */
 

@@ -72,6 +72,7 @@ SIGNATURES = {
     "moon_last_error": (C.c_char_p, [_vp]),
     "moon_sync": (_i, [_vp]),
     "moon_cleanup": (None, [_vp]),
+    "moon_set_gemm_kernel": (_i, [_vp, C.c_char_p]),
     "moon_hgemm": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _sz, _vp]),
     "moon_hgemm_trans": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _sz, _vp]),
     "moon_linear": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _i, _vp, _i, _vp]),

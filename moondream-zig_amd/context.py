@@ -111,6 +111,10 @@ class Context:
     def cleanup(self):
         self.lib.moon_cleanup(self.handle)
 
+    def set_gemm_kernel(self, name: str = ""):
+        """Measurement / test knob: the matrix-product kernel to take where the shape allows it ("" = by shape)."""
+        self.check(self.lib.moon_set_gemm_kernel(self.handle, name.encode()))
+
     # ---- resident weights
     def register_weight(self, w: np.ndarray):
         self.check(self.lib.moon_weight_register(self.handle, ptr(w), w.size))

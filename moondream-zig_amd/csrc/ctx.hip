@@ -1,4 +1,6 @@
 // Context, device memory, resident-weight registry, timers and the synthetic-data kernels.
+#include <cstring>
+
 #include "moon_internal.hpp"
 
 static thread_local std::string g_create_error;
@@ -24,6 +26,10 @@ int moon_grow(moon_ctx *ctx, GrowBuf &b, size_t bytes) {
         MOON_HIP(ctx, hipFree(b.ptr));
         b.ptr = nullptr;
         b.cap = 0;
+        if (&b == &ctx->work[1]) { // the decode-attention counters lived there: a new allocation may return the same address
+            ctx->attn_cnt_buf = nullptr;
+            ctx->attn_cnt_launches = 0;
+        }
     }
     size_t cap = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
     MOON_HIP(ctx, hipMalloc(&b.ptr, cap));
@@ -49,6 +55,7 @@ extern "C" int moon_ctx_create(int device, moon_ctx **out) {
         return moon_fail(nullptr, MOON_ENODEVICE, "device %d is %s; the kernels are built for gfx950 only", device,
                          prop.gcnArchName);
     moon_ctx *ctx = new moon_ctx();
+    if (const char *k = getenv("MOON_GEMM_KERNEL")) snprintf(ctx->gemm_kernel, sizeof ctx->gemm_kernel, "%s", k);
     ctx->device = device;
     ctx->cu_count = prop.multiProcessorCount;
     if ((e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking)) != hipSuccess ||
@@ -79,6 +86,11 @@ extern "C" void moon_cleanup(moon_ctx *ctx) {
         if (b.ptr) (void)hipFree(b.ptr);
         b = GrowBuf();
     }
+    // the per-head counters of the one-launch decode attention lived in work[1]: whatever is allocated next, at the same
+    // address or not, starts from cleared counters
+    ctx->attn_cnt_buf = nullptr;
+    ctx->attn_cnt_heads = 0;
+    ctx->attn_cnt_launches = 0;
 }
 
 extern "C" void moon_ctx_destroy(moon_ctx *ctx) {
@@ -93,6 +105,19 @@ extern "C" void moon_ctx_destroy(moon_ctx *ctx) {
     if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
+}
+
+extern "C" int moon_set_gemm_kernel(moon_ctx *ctx, const char *name) {
+    if (!ctx) return MOON_EINVAL;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    static const char *const known[] = {"", "regs", "dma", "dma256", "w114", "w212", "w221"};
+    if (!name) name = "";
+    for (const char *k : known)
+        if (!strcmp(name, k)) {
+            snprintf(ctx->gemm_kernel, sizeof ctx->gemm_kernel, "%s", name);
+            return MOON_OK;
+        }
+    return moon_fail(ctx, MOON_EINVAL, "moon_set_gemm_kernel: unknown kernel \"%s\"", name);
 }
 
 extern "C" const char *moon_last_error(const moon_ctx *ctx) { return ctx ? ctx->err.c_str() : g_create_error.c_str(); }

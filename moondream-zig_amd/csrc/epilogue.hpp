@@ -13,17 +13,16 @@ __device__ __forceinline__ float f32_round(float v) {
 }
 
 __device__ __forceinline__ float gelu_f32(float v) {
-#pragma clang fp contract(off)
-    // constants are the f16-rounded values the reference uses (ops.zig:1641-1642)
-    const float c = 0.7978515625f, alpha = 0.044708251953125f;
-    const float cube = v * v * v;
+    // constants are the f16-rounded values the reference uses (ops.zig:1641-1642): c = 0.7978515625, alpha = 0.044708251953125
     // 0.5 v (1 + tanh(u)) = v / (1 + exp(-2u)), u = c (v + alpha v^3): one exp2 and one reciprocal of the hardware (each
-    // within an ulp), no cancellation for negative v, the limits v and -0 come out exactly.  The error against the
-    // reference's f32 evaluation with a library tanh is a few f32 ulps of the result: three orders below the f16 spacing.
-    // The library tanhf costs ~45 instructions per element, which made the GELU epilogue of the vision fc1 GEMM 6 us of
-    // its 22; this form is 7 plain instructions and the two transcendental ones.
-    const float z = (c * 2.8853900817779268f) * (v + alpha * cube); // 2u / ln 2
-    const float e = __builtin_amdgcn_exp2f(-z);
+    // within an ulp), no cancellation for negative v, the limits v and -0 come out exactly.  -2u / ln 2 is taken as
+    // v * (k1 + k2 v^2) (a multiply, a fused multiply-add, a multiply): five plain instructions and the two transcendental
+    // ones per element.  The error against the reference's f32 evaluation with a library tanh is a few f32 ulps of the
+    // result: three orders below the f16 spacing.  (The library tanhf costs ~45 instructions per element, which made the
+    // GELU epilogue of the vision fc1 GEMM 6 us of its 22.)
+    constexpr float k1 = float(-0.7978515625 * 2.8853900817779268);                     // -2 c / ln 2
+    constexpr float k2 = float(-0.7978515625 * 2.8853900817779268 * 0.044708251953125); // ... * alpha
+    const float e = __builtin_amdgcn_exp2f(v * __builtin_fmaf(v * v, k2, k1));
     return f32_round(v * __builtin_amdgcn_rcpf(1.0f + e));
 }
 

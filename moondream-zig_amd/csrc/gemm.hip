@@ -19,27 +19,9 @@
 #include <atomic>
 #include <cstring>
 
-#include "epilogue.hpp"
+#include "gemm_wide.hpp"
 
 namespace {
-
-constexpr int BM = 128, BN = 128, BK = 64;
-constexpr int TILE_HALFS = 128 * BK; // one operand tile
-
-__device__ __forceinline__ int swz(int row, int granule) { return granule ^ ((row >> 1) & 7); }
-
-struct GemmArgs {
-    const half_t *A;  // [M,K]
-    const half_t *Bt; // [N,K]
-    const half_t *bias;
-    const half_t *resid; // [M,N] added after the bias for MOON_EPI_BIAS_RESID (may be C itself)
-    half_t *C;        // [M,N]
-    float *partial;   // [splits][M][N] when splits > 1
-    int M, N, K;
-    int tiles_m, tiles_n, splits, k_per_split; // k_per_split is a multiple of BK
-    int a_bytes, bt_bytes; // sizes of A and Bt (the wavefront-specialised kernels address them as buffers; < 2^31)
-    int lds_epilogue; // write the tile through LDS in full lines (needs 16-byte aligned C / bias / resid rows)
-};
 
 // Writes one wavefront's 64x64 accumulators: f16 with the epilogue, or f32 partials when K is split.
 // D[i][j] of an accumulator: i (weight row n) = 8*(v/4) + 4*(lane/32) + v%4, j (activation row m) = lane%32
@@ -316,11 +298,6 @@ constexpr int DMA_STAGES = 4;
 constexpr int DMA_THREADS = 512;
 constexpr size_t DMA_LDS_BYTES = size_t(DMA_STAGES) * 2 * TILE_HALFS * sizeof(half_t);
 
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
 template <int EPI>
 __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma_kernel(GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) half_t lds_dma[]; // [stage][operand: 0 = act (m), 1 = weight (n)][TILE_HALFS]
@@ -350,8 +327,6 @@ __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma_kernel(GemmArgs p) {
         // whose SIMD also feeds the matrix core ran at half their rate (measured 66 against 117 B/ns per CU).  Reads past
         // the end of the operand return zero, so a partial last k-tile needs no clamping (what lies beyond K is never
         // multiplied).
-        const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(p.A), 0, p.a_bytes, 0x00020000);
-        const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(p.Bt), 0, p.bt_bytes, 0x00020000);
         int off_a[4], off_w[4]; // byte offset of the granule this lane fetches, at k = 0
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -362,13 +337,19 @@ __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma_kernel(GemmArgs p) {
         }
         auto issue = [&](int kt) {
             half_t *stage = lds_dma + size_t(kt % DMA_STAGES) * 2 * TILE_HALFS;
+            // the k-tile enters through the descriptors' base and size: the range check that turns reads past the end of the
+            // operand into zeros does not see an instruction's scalar offset
             const int k_off = (k_begin + kt * BK) * 2;
+            const __amdgpu_buffer_rsrc_t rs_a =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(reinterpret_cast<const char *>(p.A)) + k_off, 0, p.a_bytes - k_off, 0x00020000);
+            const __amdgpu_buffer_rsrc_t rs_w =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(reinterpret_cast<const char *>(p.Bt)) + k_off, 0, p.bt_bytes - k_off, 0x00020000);
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (__attribute__((address_space(3))) void *)(stage + (32 * role_wave + 8 * j) * BK), 16,
-                                                         off_a[j], k_off, 0, 0);
+                                                         off_a[j], 0, 0, 0);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                    rs_w, (__attribute__((address_space(3))) void *)(stage + TILE_HALFS + (32 * role_wave + 8 * j) * BK), 16, off_w[j], k_off, 0, 0);
+                    rs_w, (__attribute__((address_space(3))) void *)(stage + TILE_HALFS + (32 * role_wave + 8 * j) * BK), 16, off_w[j], 0, 0, 0);
             }
         };
         int issued = 0; // k-tiles whose copies have been issued
@@ -935,6 +916,7 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     p.K = K;
     const size_t buf_max = (size_t(1) << 31) - 4096; // 32-bit offsets, with room for a granule past the last row
     const bool buffers_ok = size_t(M) * K * 2 < buf_max && size_t(N) * K * 2 < buf_max;
+    p.super_m = p.super_n = 1;
     p.a_bytes = buffers_ok ? int(size_t(M) * K * 2) : 0;
     p.bt_bytes = buffers_ok ? int(size_t(N) * K * 2) : 0;
     {
@@ -948,7 +930,81 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     p.tiles_n = (N + BN - 1) / BN;
     const int tiles = p.tiles_m * p.tiles_n;
     const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
-    static const char *force = getenv("MOON_GEMM_KERNEL");
+    const char *force = ctx->gemm_kernel[0] ? ctx->gemm_kernel : nullptr;
+    // The kernels with 128 x 128 accumulators per wavefront (gemm_wide.hpp)
+    const bool wide_ok = buffers_ok && K % 16 == 0 && N % 8 == 0 && p.lds_epilogue;
+    int wide = 0; // 114: 128 x 128 tiles, 212: 256 x 128, 221: 256 x 256
+    // Default: 256 x 256 tiles where they fill every CU at least once (measured 5 % faster than the 256 x 128 kernel at
+    // 4096^3); the other two arrangements measured equal to or slower than the wavefront-specialised kernels on every shape
+    // of the two models (their sum over the four wavefronts costs what their k-loop saves) and are only taken when named.
+    if (wide_ok && !force && size_t((M + 255) / 256) * ((N + 255) / 256) >= size_t(cus) && !must_fuse) wide = 221;
+    if (wide_ok && force && !strcmp(force, "w114")) wide = 114;
+    if (wide_ok && force && !strcmp(force, "w212")) wide = 212;
+    if (wide_ok && force && !strcmp(force, "w221")) wide = 221;
+    if (wide) {
+        const int tm = wide == 114 ? 128 : 256, tn = wide == 221 ? 256 : 128;
+        p.tiles_m = (M + tm - 1) / tm;
+        p.tiles_n = (N + tn - 1) / tn;
+        const int wtiles = p.tiles_m * p.tiles_n;
+        wide_super_tiles(p.tiles_m, p.tiles_n, tm, tn, &p.super_m, &p.super_n);
+        int splits = 1;
+        if (wtiles * 2 <= cus && K >= 1024) {
+            splits = cus / wtiles;
+            if (splits > K / 512) splits = K / 512;
+            if (splits > 8) splits = 8;
+            if (splits < 1) splits = 1;
+        }
+        int kps = (K + splits - 1) / splits;
+        kps = (kps + BK - 1) / BK * BK;
+        splits = (K + kps - 1) / kps;
+        p.splits = splits;
+        p.k_per_split = kps;
+        const bool ln_ok = splits > 1 && ln && N <= LN_FUSE_MAX_N && reinterpret_cast<uintptr_t>(ln->gamma) % 16 == 0 &&
+                           reinterpret_cast<uintptr_t>(ln->beta) % 16 == 0 && reinterpret_cast<uintptr_t>(ln->out) % 16 == 0 &&
+                           (!ln->add || reinterpret_cast<uintptr_t>(ln->add) % 16 == 0);
+        if (keep_partial) {
+            if (splits <= 1) return GEMM_NOT_FUSED;
+        } else if (must_fuse && !ln_ok) return GEMM_NOT_FUSED;
+        if (splits > 1) {
+            GrowBuf &ws = ctx->work[keep_partial ? 3 : 0];
+            MOON_TRY(moon_grow(ctx, ws, size_t(splits) * M * N * sizeof(float)));
+            p.partial = (float *)ws.ptr;
+        }
+        const int total = wtiles * splits;
+        const dim3 grid(((total + 7) / 8) * 8);
+        const int dev = ctx->device >= 0 && ctx->device < 64 ? ctx->device : -1;
+        // (with a split K the kernel writes partials and applies no epilogue: one instantiation serves every EPI)
+        auto go = [&](auto kern, size_t lds_bytes, std::atomic<bool> *attr_set) -> int {
+            if (dev < 0 || !attr_set[dev].load()) { // this much dynamic LDS needs the opt-in once per device and instantiation
+                MOON_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+                if (dev >= 0) attr_set[dev].store(true);
+            }
+            hipLaunchKernelGGL(kern, grid, dim3(256), lds_bytes, ctx->stream, p);
+            MOON_HIP(ctx, hipGetLastError());
+            return MOON_OK;
+        };
+        static std::atomic<bool> set114[64], set212[64], set221[64];
+        if (wide == 114) MOON_TRY(go(gemm_nt_wide_kernel<EPI, 1, 1, 4, 64>, WideCfg<1, 1, 4, 64>::LDS_BYTES, set114));
+        else if (wide == 212) MOON_TRY(go(gemm_nt_wide_kernel<EPI, 2, 1, 2, 64>, WideCfg<2, 1, 2, 64>::LDS_BYTES, set212));
+        else MOON_TRY(go(gemm_nt_wide_kernel<EPI, 2, 2, 1, 32>, WideCfg<2, 2, 1, 32>::LDS_BYTES, set221));
+        if (keep_partial) {
+            *keep_partial = p.partial;
+            *keep_splits = splits;
+            return MOON_OK;
+        }
+        if (splits > 1) {
+            const size_t mn = size_t(M) * N;
+            if (ln_ok) {
+                hipLaunchKernelGGL(splitk_reduce_ln_kernel<EPI>, dim3((unsigned)M), dim3(256), 0, ctx->stream, p.partial, bias, resid, ln->add,
+                                   ln->add_partial, ln->add_splits, ln->add_bias, C, ln->gamma, ln->beta, ln->out, M, N, splits, ln->eps);
+                *ln_done = true;
+            } else
+                hipLaunchKernelGGL(splitk_reduce8_kernel<EPI>, dim3((unsigned)((mn / 8 + 255) / 256)), dim3(256), 0, ctx->stream, p.partial, bias,
+                                   resid, C, mn, N, splits);
+            MOON_HIP(ctx, hipGetLastError());
+        }
+        return MOON_OK;
+    }
     // More 128 x 128 tiles than CUs: the 256 x 128 kernel (MOON_GEMM_KERNEL=regs|dma keeps the 128 x 128 ones).
     if (tiles > cus && buffers_ok && K % BK == 0 && N % 8 == 0 && p.lds_epilogue && !(force && (!strcmp(force, "regs") || !strcmp(force, "dma")))) {
         if (must_fuse) return GEMM_NOT_FUSED;

@@ -32,6 +32,7 @@ struct moon_ctx {
     std::mutex mu;
     std::string err;
     int cu_count = 0;
+    char gemm_kernel[8] = ""; // moon_set_gemm_kernel / MOON_GEMM_KERNEL: a product kernel to take where the shape allows it ("": by shape)
     // staging for host-pointer ops: a, b, c, bias/aux, mask
     GrowBuf stage[6];
     // kernel workspaces (split-K partials, attention partials, transposed B)

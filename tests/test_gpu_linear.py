@@ -171,3 +171,34 @@ def test_registered_weight_in_hgemm_layout(moon, O, ctx):
     ctx.unregister_weight(w)
     assert O.rel_frobenius(doubled, O.hgemm(a, w)) <= TOL
     assert np.array_equal(moon.hgemm.matmul(a, w, ctx=ctx), doubled)
+
+
+# The product kernels that the default choice takes only for some shapes (or never), each named through the context's knob:
+# the same products to the same bar.  Shapes cover ragged tile edges, a partial last k-tile (K % 64 == 16, 32, 48), K short
+# of the stage count, the split K, and every epilogue.
+@pytest.mark.parametrize("kernel", ["w114", "w212", "w221", "dma", "dma256", "regs"])
+def test_named_product_kernels(moon, O, ctx, kernel):
+    L = moon._lib
+    shapes = [(200, 320, 264, "bias"), (300, 80, 520, "none"), (729, 1152, 1152, "bias"), (513, 144, 776, "bias_gelu"),
+              (130, 2096, 136, "bias"), (257, 48, 264, "none")]
+    ctx.set_gemm_kernel(kernel)
+    try:
+        for M, K, N, epi in shapes:
+            a = O.fill_normal_f16((M, K), 0, 0, 1.0)
+            w = O.fill_normal_f16((N, K), 0, 1, 0.05)
+            b = O.fill_normal_f16((N,), 0, 2, 0.1)
+            code = {"none": L.EPI_NONE, "bias": L.EPI_BIAS, "bias_gelu": L.EPI_BIAS_GELU}[epi]
+            got = np.empty((M, N), dtype=np.float16)
+            ctx.check(ctx.lib.moon_linear(ctx.handle, a.ctypes.data, M, K, w.ctypes.data, N, L.B_NK, b.ctypes.data if epi != "none" else None, code,
+                                          got.ctypes.data))
+            ref = O.hgemm_trans(a, w)
+            if epi != "none":
+                ref = O.bias_add(ref, b)
+            if epi == "bias_gelu":
+                ref = O.gelu(ref)
+            err = O.rel_frobenius(got, ref)
+            assert err <= TOL, (kernel, M, K, N, epi, err)
+    finally:
+        ctx.set_gemm_kernel("")
+    with pytest.raises(moon.InvalidArgument):
+        ctx.set_gemm_kernel("nonesuch")
