@@ -155,8 +155,6 @@ def profile_decode_kernels(model, us_per_token, mode=None):
     An event interval is the kernel plus the command processor's handling of the two events; that overhead is taken
     from the same run: (sum of all intervals of a token - the un-instrumented time per token) / launches per token,
     and subtracted from every interval."""
-    if mode == 1:  # the persistent kernel cannot be timed per launch: profile the default kernels instead
-        model.set_decode_mode(0)
     _, prof = model.greedy_profile(PROFILE_STEPS)
     kv_mid = model.position - PROFILE_STEPS / 2
     # algorithmic bytes per launch: weights and biases once, activations in and out once
@@ -396,7 +394,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run 8 plain 256 MiB copies (copy16_kernel) as the known-traffic yardstick for a counter run")
     ap.add_argument("--decode-mode", type=int, default=None,
-                    help="0: one kernel per layer (default), 1: persistent kernel, 2: three kernels per layer, 3: two kernels per layer")
+                    help="0: one kernel per layer (default), 2: three kernels per layer, 3: two kernels per layer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives or sharding exist); use --gpus 1")

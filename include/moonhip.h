@@ -270,6 +270,13 @@ int moon_text_reset(moon_text_model *m);
 /* text_encoder + text_decoder over n_ids tokens appended at the current cache length
  * (text_model.zig:106-180); n_ids == 1 runs the decode kernels. */
 int moon_text_forward(moon_text_model *m, const uint32_t *ids, size_t n_ids);
+/* TextModel.text_decoder as the reference's host calls it (text_model.zig:139-180; moondream.zig:296-327): the input is
+ * rows of embeddings [n_rows, dim] in host memory (the image features and the prompt's embeddings side by side, later one
+ * row per token), appended at the session's position.  moon_text_hidden then gives `output`. */
+int moon_text_forward_embeds(moon_text_model *m, const moon_f16 *embeds, size_t n_rows);
+/* TextModel.text_encoder (text_model.zig:106-137): embeds[n_ids, dim] = rows ids[i] of the embedding table, to host
+ * memory.  Does not touch the session's position or cache.  error.TokenIdOutOfBounds -> MOON_ETOKEN. */
+int moon_text_embed(moon_text_model *m, const uint32_t *ids, size_t n_ids, moon_f16 *embeds);
 /* lm_head of the last position of the previous forward (text_model.zig:325-345) -> logits[vocab]. */
 int moon_text_logits(moon_text_model *m, moon_f16 *logits);
 /* n_steps of: lm_head -> argmax -> text_encoder([id]) -> text_decoder (moondream.zig:323-368),
@@ -280,6 +287,20 @@ int moon_text_greedy(moon_text_model *m, size_t n_steps, uint32_t *out_ids);
  * logits never leave HBM.  u[n_steps] holds the numbers the reference would draw from its PRNG, one per step
  * (ignored, and may be NULL, for MOON_SAMPLE_GREEDY, which runs moon_text_greedy). */
 int moon_text_sample(moon_text_model *m, const moon_sampling_config *cfg, const float *u, size_t n_steps, uint32_t *out_ids);
+/* The generation loop of moondream.zig:323-368 (moonchat.zig:597-603) on the device: up to max_tokens steps of
+ * {lm_head, sampling.sample (cfg == NULL or MOON_SAMPLE_GREEDY: arg-max), text_encoder of the new token, text_decoder},
+ * ended early by the end-of-sequence token (moondream.zig:341: that token is not part of the output) or by the last cache
+ * position (moondream.zig:324).  out_ids[max_tokens] receives the tokens, *n_out their number.  The host looks at the
+ * device's state every 8 steps, so at most 8 steps are queued behind the stop; after a stop by the end-of-sequence token
+ * the session needs a moon_text_forward before the next loop (the queued steps have overwritten its hidden state).
+ * u[max_tokens]: as in moon_text_sample. */
+int moon_text_generate(moon_text_model *m, const moon_sampling_config *cfg, const float *u, size_t max_tokens, uint32_t eos_token,
+                       uint32_t *out_ids, size_t *n_out);
+/* One step of that loop for a host that keeps the loop itself, as the reference does (moondream.zig:333-337:
+ * text_model.lm_head + sampling.sample on the last position of the latest moon_text_forward): the token comes back, the
+ * logits stay on the device.  The host then feeds it with moon_text_forward(m, &token, 1).  u: the reference's one draw
+ * from its PRNG (ignored for the arg-max). */
+int moon_text_next_token(moon_text_model *m, const moon_sampling_config *cfg, float u, uint32_t *token);
 /* moon_text_greedy (decode modes 0, 2, 3) with a HIP event pair (on the library's stream) around every kernel launch:
  * avg_us[6] / launches[6] = average event interval and launch count of {LayerNorm+qkv+fc1 (in mode 0 the whole layer,
  * in mode 3 including the attention), rope+append+attention (mode 2 only), out_proj+fc2+residual (modes 2, 3), final
@@ -292,14 +313,9 @@ int moon_text_sample(moon_text_model *m, const moon_sampling_config *cfg, const 
 int moon_text_greedy_profile(moon_text_model *m, size_t n_steps, uint32_t *out_ids, float *avg_us, size_t *launches);
 /* How moon_text_greedy runs a decoder layer: 0 (default) = one kernel per layer (its workgroups hand qkv, fc1 and the
  * attention output to each other through counters, with bounded waits) where the device can hold enough of that
- * kernel's workgroups at once, else as mode 3 or 2; 1 = one persistent kernel for the whole greedy loop (all workgroups
- * co-resident, device-wide barriers between phases); 2 = three kernels per layer and no waits inside kernels;
- * 3 = two kernels per layer (LayerNorm + qkv + fc1 + attention; out_proj + fc2 + residual).  Modes 0-3 produce the same bits.
- * 4 = the streaming kernel: the whole greedy loop as one launch that keeps every compute unit reading weights through LDS
- * rings while two workgroups per unit exchange q/k/v, attention partials, partial sums of out_proj / fc2 and the hidden
- * state through tagged words (default configuration on a 256-unit device only; out_proj and fc2 are summed per workgroup and
- * then over workgroups, so its logits differ from the other modes' in the last bits: same tolerance, same token ids in
- * the tests).  A wait that expires makes the call return MOON_EHIP. */
+ * kernel's workgroups at once, else as mode 3 or 2; 2 = three kernels per layer and no waits inside kernels;
+ * 3 = two kernels per layer (LayerNorm + qkv + fc1 + attention; out_proj + fc2 + residual).  All modes produce the same
+ * bits.  A wait that expires makes the call return MOON_EHIP.  No counterpart in the reference. */
 int moon_text_set_decode_mode(moon_text_model *m, int mode);
 /* After a MOON_EHIP from moon_text_greedy / moon_text_sample caused by an expired wait inside a fused decode kernel the
  * session refuses further forward / greedy / sample calls until moon_text_reset: workgroups that gave up may have skipped
@@ -366,6 +382,10 @@ int moon_vision_io_attach_synthetic(moon_vision_model *m, const moon_vision_io_c
  * reference does (attention_block takes q_len = B * M, :273-329).  MOON_EINVAL if nothing is attached. */
 int moon_vision_encode_image(moon_vision_model *m, const moon_f16 *patches, moon_f16 *out);
 int moon_vision_encode_image_dev(moon_vision_model *m, const void *patches, void *out);
+/* VisionModel.vision_encoder (vision_model.zig:204-271) behind its rearrangeBCHWtoBTC: patches[2 * tokens, patch_dim] ->
+ * out[2 * tokens, dim] = patch embedding + bias + positional embedding, the encoder blocks on all rows as one sequence, the
+ * final LayerNorm (what encode_image then splits, concatenates and projects). */
+int moon_vision_encoder(moon_vision_model *m, const moon_f16 *patches, moon_f16 *out);
 /* VisionModel.encode_image from the resized image on (vision_model.zig:129-229): image[side, side, 3] as stbir left it
  * (side = sqrt(tokens) * sqrt(patch_dim / 3), 378 for the default configuration), normalised and cut into patches on the
  * device as moon_image_patches does, then moon_vision_encode_image's path. */
@@ -399,14 +419,13 @@ int moon_bin_vision_io_weights(const moon_bin *bin, const moon_vision_config *cf
  * diagnostic aids, read once per process (the first call that looks at them fixes the value for every context):
  *   MOON_DECODE_TRACE=1            text sessions record per-workgroup time stamps of the last layer launch of a greedy call
  *                                  and print a per-role timeline to stderr (allocated at session creation)
- *   MOON_STREAM_DEBUG=n            decode mode 4 only: switches parts of the streaming kernel off (timing experiments; wrong results)
  *   MOON_LAYER_OUT_CHUNK=1|2|4|8|16  decode mode 0: 1 KiB pieces of an fc2 row an output wavefront requests before it waits (default 4)
  *   MOON_LAYER_QKV_WGS=n           decode mode 0: workgroups that take qkv rows (default: the attention and output workgroups)
  *   MOON_LAYER_FC1_OUT_ROWS=n      decode mode 0: fc1 rows per output wavefront (default: half an fc1-only wavefront's share)
  *   MOON_LAYER_FC1_GROUP=1|2       decode mode 0: fc1 rows a wavefront requests together (default 1)
  *   MOON_GEMM_KERNEL=regs|dma|dma256|w114|w212|w221  forces one of the MFMA product kernels where the shape allows it (default: by shape)
  *   MOON_GEMM_EPILOGUE=direct      the product kernels store their tile without the pass through LDS (default: through LDS)
- * Every setting gives the same results (bit for bit, MOON_STREAM_DEBUG aside); only the time changes. */
+ * Every setting gives the same results, bit for bit; only the time changes. */
 
 #ifdef __cplusplus
 }

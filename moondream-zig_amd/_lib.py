@@ -119,6 +119,10 @@ SIGNATURES = {
     "moon_text_logits": (_i, [_vp, _vp]),
     "moon_text_greedy": (_i, [_vp, _sz, _vp]),
     "moon_text_sample": (_i, [_vp, _vp, _vp, _sz, _vp]),
+    "moon_text_forward_embeds": (_i, [_vp, _vp, _sz]),
+    "moon_text_embed": (_i, [_vp, _vp, _sz, _vp]),
+    "moon_text_generate": (_i, [_vp, _vp, _vp, _sz, _u32, _vp, C.POINTER(_sz)]),
+    "moon_text_next_token": (_i, [_vp, _vp, _f, C.POINTER(_u32)]),
     "moon_text_greedy_profile": (_i, [_vp, _sz, _vp, _vp, _vp]),
     "moon_text_set_decode_mode": (_i, [_vp, _i]),
     "moon_text_debug_raise_wait_error": (_i, [_vp]),
@@ -135,6 +139,7 @@ SIGNATURES = {
     "moon_vision_io_attach": (_i, [_vp, C.POINTER(VisionIoConfig), C.POINTER(VisionIoWeights)]),
     "moon_vision_io_attach_synthetic": (_i, [_vp, C.POINTER(VisionIoConfig), _u64, _f]),
     "moon_vision_encode_image": (_i, [_vp, _vp, _vp]),
+    "moon_vision_encoder": (_i, [_vp, _vp, _vp]),
     "moon_vision_encode_image_dev": (_i, [_vp, _vp, _vp]),
     "moon_vision_encode_image_u8": (_i, [_vp, _vp, _vp]),
     "moon_bin_open": (_i, [C.c_char_p, _pp, C.c_char_p, _sz]),

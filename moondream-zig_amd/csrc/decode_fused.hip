@@ -272,12 +272,7 @@ __global__ __launch_bounds__(256) void decode_lm_head_kernel(LmHeadArgs a) {
     if (tid == 0) {
         for (int w = 1; w < 4; w++) argmax_merge(best, best_i, s_best[w], s_idx[w]);
         const uint32_t tok = best_i == 0x7fffffff ? 0u : (uint32_t)best_i;
-        a.state[2] = tok;
-        if (a.out_ids) {
-            a.out_ids[a.state[1]] = tok;
-            a.state[1] += 1;
-        }
-        a.state[0] += a.bump;
+        record_token(a.state, a.out_ids, tok, a.bump);
     }
 }
 
@@ -778,11 +773,7 @@ __global__ __launch_bounds__(1024) void argmax_record_kernel(const half_t *__res
             }
         const float first = (float)logits[0];
         const uint32_t tok = (idx == 0x7fffffff || first != first) ? 0u : (uint32_t)idx; // a NaN at index 0 is never displaced
-        state[2] = tok;
-        if (out_ids) {
-            out_ids[state[1]] = tok;
-            state[1] += 1;
-        }
+        record_token(state, out_ids, tok, 0u);
     }
 }
 

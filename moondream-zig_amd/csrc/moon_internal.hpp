@@ -68,6 +68,28 @@ int moon_grow(moon_ctx *ctx, GrowBuf &b, size_t bytes);
         if (_rc != MOON_OK) return _rc; \
     } while (0)
 
+// Bookkeeping of the on-device generation loop (moondream.zig:323-368), one thread at the end of the kernel that picked the
+// token.  state: [0] position (KV length), [1] tokens recorded so far, [2] current token, [3] 1 once the end-of-sequence
+// token has come up, [4] that token's id + 1 (0: none).  The position moves on by `bump` (the append of the previous
+// step's token); the end-of-sequence token is neither recorded nor does anything move after it (moondream.zig:341 breaks
+// out of the loop there): the launches that the host had already queued behind it keep appending to the one position after
+// the last valid one, which the session never reads.
+#if defined(__HIPCC__)
+__device__ __forceinline__ void record_token(uint32_t *state, uint32_t *out_ids, uint32_t tok, uint32_t bump) {
+    if (state[3]) return;
+    state[0] += bump;
+    state[2] = tok;
+    if (state[4] == tok + 1u) {
+        state[3] = 1u;
+        return;
+    }
+    if (out_ids) {
+        out_ids[state[1]] = tok;
+        state[1] += 1;
+    }
+}
+#endif
+
 // ---- kernel launchers (all asynchronous on ctx->stream, device pointers) ----
 
 // y[N] = epi(x[K] . W[N,K]); K % 8 == 0 takes the 128-bit path.

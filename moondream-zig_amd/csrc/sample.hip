@@ -665,12 +665,7 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs p) {
     }
     if (t == 0) {
         if (p.out) p.out[0] = (uint32_t)token;
-        if (p.state) {
-            p.state[2] = (uint32_t)token;
-            p.out_ids[p.state[1]] = (uint32_t)token;
-            p.state[1] += 1;
-            p.state[0] += p.bump_pos; // the position moves on here, as it does in the fused LM-head + arg-max kernel
-        }
+        if (p.state) record_token(p.state, p.out_ids, (uint32_t)token, p.bump_pos); // as the fused LM-head + arg-max kernel does
     }
 }
 

@@ -5,36 +5,10 @@
 // Activations and the cache never leave the device; a decode step enqueues kernels only (token id and position
 // are read from device memory), so the loop needs no host synchronisation until the ids are fetched.
 #include "moon_internal.hpp"
-#include "decode_stream.hpp"
 
 #include <cstdlib>
 #include <algorithm>
 #include <vector>
-
-// persistent decode kernel (text_decode_fused.hip)
-struct DecodeParams {
-    const half_t *wte, *ln_w, *ln_b, *qkv_w, *qkv_b, *out_w, *out_b, *fc1_w, *fc1_b, *fc2_w, *fc2_b, *lin_w, *lin_b, *lno_w, *lno_b;
-    half_t *cache_k, *cache_v;
-    const float *freqs;
-    half_t *hidden;
-    const half_t *hidden_first;
-    half_t *qkv;
-    half_t *fc1;
-    half_t *attn;
-    half_t *logits;
-    float *attn_partial;
-    float *amax_val;
-    int *amax_idx;
-    uint32_t *out_ids;
-    uint32_t *sync;
-    int d, ffn, H, L, V, rot_dim, max_seq, pos0, n_steps;
-    float eps;
-    long long *trace;
-};
-int decode_persistent_groups(moon_ctx *ctx, size_t d, size_t ffn, int *groups, size_t *shmem);
-int launch_decode_persistent(moon_ctx *ctx, DecodeParams &p, int groups, size_t shmem);
-size_t decode_persistent_sync_words();
-size_t decode_persistent_error_word();
 
 // fused decode kernels (decode_fused.hip)
 bool decode_fused_supported(size_t d, size_t ffn);
@@ -90,17 +64,11 @@ struct moon_text_model {
            *fc1 = nullptr, *mlp = nullptr, *logits = nullptr, *ln_last = nullptr;
     uint32_t *ids_dev = nullptr;   // [max_seq] prompt ids / generated ids
     float *u_dev = nullptr;        // [max_seq] the sampling loop's random numbers, one per step
-    uint32_t *state_dev = nullptr; // [0] = position (KV length), [1] = step counter, [2] = current token
+    uint32_t *state_dev = nullptr; // [0] position (KV length), [1] tokens recorded, [2] current token, [3] stopped, [4] eos id + 1 (record_token)
     size_t cur_len = 0, last_n = 0;
     bool cache_invalid = false;    // a fused decode kernel gave up on a wait: positions may be missing from the cache until moon_text_reset
-    // persistent decode kernel state
-    int decode_mode = 0;           // 0: a few fused kernels per layer (default); 1: one persistent kernel for the whole greedy loop
-    int groups = 0;                // co-resident workgroups of the persistent kernel (0: unavailable)
-    size_t persistent_shmem = 0;
+    int decode_mode = 0;           // 0: one kernel per layer where the device holds it (default); 2: three kernels per layer; 3: two
     float *attn_partial = nullptr; // [H][8][66]
-    float *amax_val = nullptr;     // [groups]
-    int *amax_idx = nullptr;       // [groups]
-    uint32_t *sync_dev = nullptr;  // barrier state of the persistent kernel
     // fused per-layer decode kernels
     bool fused = false;              // shape supported by decode_fused.hip
     uint32_t *head_count = nullptr;  // [L][H] "splits finished" counters, monotonically increasing
@@ -114,14 +82,6 @@ struct moon_text_model {
     std::vector<uint32_t> layer_launches;
     uint32_t *lm_exchange = nullptr;  // arg-max pairs of the LM head's workgroups, then their counter (monotonic)
     uint32_t lm_launches = 0;
-    // streaming decode kernel (decode mode 4): the whole greedy loop as one launch, decode_stream.hip
-    bool stream = false;              // shape and device supported
-    half_t *fc2_wt = nullptr, *out_wt = nullptr; // [L][ffn][d], [L][d][d]: transposed copies made at creation
-    half_t *stream_arena = nullptr;   // one allocation holding qkv_w, fc1_w, fc2_wt, out_wt, lin_w (the kernel addresses them with 32-bit offsets)
-    size_t stream_arena_bytes = 0;
-    uint32_t *stream_sync = nullptr;  // hid_t | qkv_t | ap_t | rp_t | am_t | error word, see stream_layout()
-    uint32_t stream_gen = 0;          // tags used so far on those buffers
-    long long *stream_trace = nullptr;
     long long *layer_trace = nullptr; // [grid][8] stamps of the most recent layer launch when MOON_DECODE_TRACE is set
     struct StepProfiler *prof = nullptr;  // set only inside moon_text_greedy_profile
     std::vector<void *> allocs;
@@ -129,15 +89,20 @@ struct moon_text_model {
 
 namespace {
 
-__global__ void record_token_kernel(uint32_t *state, uint32_t *out_ids) {
-    // state[2] was just written by the arg-max kernel
-    out_ids[state[1]] = state[2];
-    state[1] += 1;
+__global__ void bump_pos_kernel(uint32_t *state) {
+    if (!state[3]) state[0] += 1;
 }
-__global__ void bump_pos_kernel(uint32_t *state) { state[0] += 1; }
+// two neighbouring words (the loop's position and step count; also used to raise an error word next to a counter's tail)
 __global__ void set_state_kernel(uint32_t *state, uint32_t pos, uint32_t step) {
     state[0] = pos;
     state[1] = step;
+}
+// the generation loop's state before its first step (record_token): position, no tokens yet, not stopped, eos id + 1 (0: none)
+__global__ void start_loop_kernel(uint32_t *state, uint32_t pos, uint32_t eos_plus1) {
+    state[0] = pos;
+    state[1] = 0;
+    state[3] = 0;
+    state[4] = eos_plus1;
 }
 
 int dalloc(moon_text_model *m, size_t bytes, void **p) {
@@ -164,48 +129,20 @@ int check_cfg(moon_ctx *ctx, const moon_text_config *c) {
     return MOON_OK;
 }
 
-// 32-bit word offsets of the streaming kernel's exchange buffers inside stream_sync (the 64-bit ones on 8-byte boundaries)
-struct StreamLayout {
-    size_t hid, qkv, ap, rp, rp_flag, am, err, words;
-};
-StreamLayout stream_layout() {
-    StreamLayout o;
-    o.hid = 0;
-    o.qkv = o.hid + STREAM_HID_WORDS;
-    o.ap = o.qkv + STREAM_QKV_WORDS;
-    o.rp = o.ap + 2 * STREAM_AP_WORDS;
-    o.rp_flag = o.rp + STREAM_RP_FLOATS;
-    o.am = o.rp_flag + STREAM_RP_FLAGS;
-    o.err = o.am + 2 * STREAM_AM_WORDS + 32; // a line of its own
-    o.words = o.err + 32;
-    return o;
-}
-
 int alloc_all(moon_text_model *m) {
     const Sizes z = sizes(m->cfg);
-    m->stream = decode_stream_supported(m->ctx, z.d, z.ffn, z.H, z.D, z.S, z.L, z.V);
-    if (m->stream) { // the matrices the streaming kernel reads, in one allocation
-        const size_t n_qkv = z.L * 3 * z.d * z.d, n_fc = z.L * z.ffn * z.d, n_out = z.L * z.d * z.d, n_lin = z.V * z.d;
-        m->stream_arena_bytes = (n_qkv + 2 * n_fc + n_out + n_lin) * sizeof(half_t);
-        MOON_TRY(dalloc_t(m, n_qkv + 2 * n_fc + n_out + n_lin, &m->stream_arena));
-        m->qkv_w = m->stream_arena;
-        m->fc1_w = m->qkv_w + n_qkv;
-        m->fc2_wt = m->fc1_w + n_fc;
-        m->out_wt = m->fc2_wt + n_fc;
-        m->lin_w = m->out_wt + n_out;
-    }
     MOON_TRY(dalloc_t(m, z.V * z.d, &m->wte));
     MOON_TRY(dalloc_t(m, z.L * z.d, &m->ln_w));
     MOON_TRY(dalloc_t(m, z.L * z.d, &m->ln_b));
-    if (!m->stream) MOON_TRY(dalloc_t(m, z.L * 3 * z.d * z.d, &m->qkv_w));
+    MOON_TRY(dalloc_t(m, z.L * 3 * z.d * z.d, &m->qkv_w));
     MOON_TRY(dalloc_t(m, z.L * 3 * z.d, &m->qkv_b));
     MOON_TRY(dalloc_t(m, z.L * z.d * z.d, &m->out_w));
     MOON_TRY(dalloc_t(m, z.L * z.d, &m->out_b));
-    if (!m->stream) MOON_TRY(dalloc_t(m, z.L * z.ffn * z.d, &m->fc1_w));
+    MOON_TRY(dalloc_t(m, z.L * z.ffn * z.d, &m->fc1_w));
     MOON_TRY(dalloc_t(m, z.L * z.ffn, &m->fc1_b));
     MOON_TRY(dalloc_t(m, z.L * z.d * z.ffn, &m->fc2_w));
     MOON_TRY(dalloc_t(m, z.L * z.d, &m->fc2_b));
-    if (!m->stream) MOON_TRY(dalloc_t(m, z.V * z.d, &m->lin_w));
+    MOON_TRY(dalloc_t(m, z.V * z.d, &m->lin_w));
     MOON_TRY(dalloc_t(m, z.V, &m->lin_b));
     MOON_TRY(dalloc_t(m, z.d, &m->lno_w));
     MOON_TRY(dalloc_t(m, z.d, &m->lno_b));
@@ -224,15 +161,9 @@ int alloc_all(moon_text_model *m) {
     MOON_TRY(dalloc_t(m, z.d, &m->ln_last));
     MOON_TRY(dalloc_t(m, z.S, &m->ids_dev));
     MOON_TRY(dalloc_t(m, z.S, &m->u_dev));
-    MOON_TRY(dalloc_t(m, 4, &m->state_dev));
-    if (z.d % 8 == 0 && z.ffn % 8 == 0) {
-        int rc = decode_persistent_groups(m->ctx, z.d, z.ffn, &m->groups, &m->persistent_shmem);
-        if (rc != MOON_OK || z.d > size_t(16) * m->groups) m->groups = 0;
-    }
+    MOON_TRY(dalloc_t(m, 8, &m->state_dev));
+    MOON_TRY(launch_fill_uniform_u32(m->ctx, m->state_dev, 8, 0, 0, 1)); // zeros
     MOON_TRY(dalloc_t(m, z.H * 8 * 66, &m->attn_partial));
-    MOON_TRY(dalloc_t(m, m->groups + 1, &m->amax_val));
-    MOON_TRY(dalloc_t(m, 2 * m->groups + 2, &m->amax_idx));
-    MOON_TRY(dalloc_t(m, decode_persistent_sync_words(), &m->sync_dev));
     m->fused = decode_fused_supported(z.d, z.ffn);
     MOON_TRY(dalloc_t(m, z.L * z.H, &m->head_count));
     MOON_TRY(launch_fill_uniform_u32(m->ctx, m->head_count, z.L * z.H, 0, 0, 1)); // zeros
@@ -248,15 +179,7 @@ int alloc_all(moon_text_model *m) {
     m->layer_launches.assign(z.L, 0);
     MOON_TRY(dalloc_t(m, decode_lm_head_words(m->ctx), &m->lm_exchange));
     MOON_TRY(launch_fill_uniform_u32(m->ctx, m->lm_exchange, decode_lm_head_words(m->ctx), 0, 0, 1)); // zeros
-    if (m->stream) {
-        MOON_TRY(dalloc_t(m, stream_layout().words, &m->stream_sync));
-        MOON_TRY(launch_fill_uniform_u32(m->ctx, m->stream_sync, stream_layout().words, 0, 0, 1)); // zeros
-    }
     if (getenv("MOON_DECODE_TRACE")) {
-        if (m->stream) {
-            MOON_TRY(dalloc_t(m, z.L * size_t(STREAM_GRID) * 8, &m->stream_trace));
-            MOON_TRY(launch_fill_uniform_u32(m->ctx, (uint32_t *)m->stream_trace, z.L * size_t(STREAM_GRID) * 16, 0, 0, 1));
-        }
         MOON_TRY(dalloc_t(m, size_t(4096) * 8, &m->layer_trace));
         MOON_TRY(launch_fill_uniform_u32(m->ctx, (uint32_t *)m->layer_trace, size_t(4096) * 16, 0, 0, 1));
     }
@@ -285,23 +208,10 @@ int clear_sync_state(moon_text_model *m) {
     MOON_TRY(launch_fill_uniform_u32(ctx, m->front_sync, z.L * z.H * 32 + 1, 0, 0, 1));
     MOON_TRY(launch_fill_uniform_u32(ctx, m->layer_sync, z.L * m->layer_sync_words + 1, 0, 0, 1));
     MOON_TRY(launch_fill_uniform_u32(ctx, m->lm_exchange, decode_lm_head_words(ctx), 0, 0, 1));
-    if (m->stream) MOON_TRY(launch_fill_uniform_u32(ctx, m->stream_sync, stream_layout().words, 0, 0, 1));
-    m->stream_gen = 0;
     m->attn_launches.assign(z.L, 0);
     m->front_launches.assign(z.L, 0);
     m->layer_launches.assign(z.L, 0);
     m->lm_launches = 0;
-    return MOON_OK;
-}
-
-// The streaming kernel reads fc2 and out_proj by input column: transposed copies, made once when the weights are in place.
-int prepare_stream(moon_text_model *m) {
-    if (!m->stream) return MOON_OK;
-    const Sizes z = sizes(m->cfg);
-    for (size_t l = 0; l < z.L; l++) {
-        MOON_TRY(launch_transpose(m->ctx, m->fc2_w + l * z.d * z.ffn, m->fc2_wt + l * z.ffn * z.d, z.d, z.ffn));
-        MOON_TRY(launch_transpose(m->ctx, m->out_w + l * z.d * z.d, m->out_wt + l * z.d * z.d, z.d, z.d));
-    }
     return MOON_OK;
 }
 
@@ -345,7 +255,7 @@ int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool p
     if (n == 1 && m->fused) {
         // three kernels: LN + qkv + fc1;  rope + append + attention (+ merge);  out_proj + fc2 + both residual adds
         const half_t *x = token_dev ? m->wte : m->hidden;
-        const int mode = m->decode_mode == 4 ? 0 : m->decode_mode; // the streaming kernel is a loop; single steps take the per-layer kernels
+        const int mode = m->decode_mode;
         if (m->whole_layer && mode == 0) {
             // one kernel for the layer
             const uint32_t head_target = ++m->attn_launches[layer] * 8u;
@@ -484,7 +394,6 @@ extern "C" int moon_text_model_create(moon_ctx *ctx, const moon_text_config *cfg
     up(m->lin_b, w->t_linear_b, z.V);
     up(m->lno_w, w->t_ln_out_w, z.d);
     up(m->lno_b, w->t_ln_out_b, z.d);
-    if (rc == MOON_OK) rc = prepare_stream(m);
     if (rc == MOON_OK) {
         hipError_t e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) rc = moon_fail(ctx, MOON_EHIP, "weight upload sync: %s", hipGetErrorString(e));
@@ -532,7 +441,6 @@ extern "C" int moon_text_model_create_synthetic(moon_ctx *ctx, const moon_text_c
     rnd(m->lin_b, z.V, 12);
     cst(m->lno_w, z.d, 1.0f);
     cst(m->lno_b, z.d, 0.0f);
-    if (rc == MOON_OK) rc = prepare_stream(m);
     if (rc == MOON_OK) {
         hipError_t e = hipStreamSynchronize(ctx->stream);
         if (e != hipSuccess) rc = moon_fail(ctx, MOON_EHIP, "synthetic weights: %s", hipGetErrorString(e));
@@ -570,6 +478,33 @@ extern "C" int moon_text_reset(moon_text_model *m) {
 
 extern "C" size_t moon_text_position(const moon_text_model *m) { return m ? m->cur_len : 0; }
 
+// n rows already in m->hidden: the layers, the bookkeeping and, for a single row, the fused kernels' error words
+static int forward_rows_locked(moon_text_model *m, size_t n_ids) {
+    moon_ctx *ctx = m->ctx;
+    for (size_t l = 0; l < m->cfg.n_layers; l++) MOON_TRY(layer_forward(m, l, n_ids, m->cur_len, false, nullptr, n_ids > 1));
+    m->cur_len += n_ids;
+    m->last_n = n_ids;
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->state_dev, (uint32_t)m->cur_len, 0u);
+    MOON_HIP(ctx, hipGetLastError());
+    // a single token takes the fused decode kernels, whose waits between workgroups are bounded: look at their error words
+    uint32_t wait_error[2] = {0, 0};
+    if (n_ids == 1 && m->fused) {
+        MOON_HIP(ctx, hipMemcpyAsync(&wait_error[0], m->layer_sync + m->cfg.n_layers * m->layer_sync_words, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                     ctx->stream));
+        MOON_HIP(ctx, hipMemcpyAsync(&wait_error[1], m->front_sync + m->cfg.n_layers * m->cfg.n_heads * 32, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                     ctx->stream));
+    }
+    MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (wait_error[0] || wait_error[1]) { // as in the generation loop: the token's cache row may be missing
+        m->cur_len -= n_ids;
+        m->cache_invalid = true;
+        m->last_n = 0;
+        (void)clear_sync_state(m);
+        return moon_fail(ctx, MOON_EHIP, "fused decode kernel: a wait between its phases timed out; the session needs moon_text_reset");
+    }
+    return MOON_OK;
+}
+
 extern "C" int moon_text_forward(moon_text_model *m, const uint32_t *ids, size_t n_ids) {
     if (!m) return MOON_EINVAL;
     moon_ctx *ctx = m->ctx;
@@ -584,11 +519,39 @@ extern "C" int moon_text_forward(moon_text_model *m, const uint32_t *ids, size_t
     MOON_HIP(ctx, hipSetDevice(ctx->device));
     MOON_HIP(ctx, hipMemcpyAsync(m->ids_dev, ids, n_ids * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
     MOON_TRY(launch_embed(ctx, m->wte, m->ids_dev, m->hidden, n_ids, m->cfg.dim));
-    for (size_t l = 0; l < m->cfg.n_layers; l++) MOON_TRY(layer_forward(m, l, n_ids, m->cur_len, false, nullptr, n_ids > 1));
-    m->cur_len += n_ids;
-    m->last_n = n_ids;
-    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->state_dev, (uint32_t)m->cur_len, 0u);
-    MOON_HIP(ctx, hipGetLastError());
+    return forward_rows_locked(m, n_ids);
+}
+
+extern "C" int moon_text_forward_embeds(moon_text_model *m, const moon_f16 *embeds, size_t n_rows) {
+    if (!m) return MOON_EINVAL;
+    moon_ctx *ctx = m->ctx;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (!embeds && n_rows) return moon_fail(ctx, MOON_EINVAL, "text_forward_embeds: null input");
+    if (!n_rows) return moon_fail(ctx, MOON_EINVAL_DIM, "text_forward_embeds: empty input (InvalidInputShape)");
+    if (m->cache_invalid) return moon_fail(ctx, MOON_EHIP, "text_forward_embeds: an earlier decode call failed; call moon_text_reset first");
+    if (m->cur_len + n_rows > m->cfg.max_seq)
+        return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "text_forward_embeds: %zu + %zu rows > max_seq %zu (SequenceTooLong)", m->cur_len, n_rows, m->cfg.max_seq);
+    MOON_HIP(ctx, hipSetDevice(ctx->device));
+    MOON_HIP(ctx, hipMemcpyAsync(m->hidden, embeds, n_rows * m->cfg.dim * sizeof(moon_f16), hipMemcpyHostToDevice, ctx->stream));
+    return forward_rows_locked(m, n_rows);
+}
+
+extern "C" int moon_text_embed(moon_text_model *m, const uint32_t *ids, size_t n_ids, moon_f16 *embeds) {
+    if (!m) return MOON_EINVAL;
+    moon_ctx *ctx = m->ctx;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if ((!ids || !embeds) && n_ids) return moon_fail(ctx, MOON_EINVAL, "text_embed: null argument");
+    if (n_ids > m->cfg.max_seq) return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "text_embed: %zu ids > seq_len %zu (SequenceTooLong)", n_ids, m->cfg.max_seq);
+    for (size_t i = 0; i < n_ids; i++)
+        if (ids[i] >= m->cfg.vocab) return moon_fail(ctx, MOON_ETOKEN, "text_embed: token id %u >= vocab %zu (TokenIdOutOfBounds)", ids[i], m->cfg.vocab);
+    if (!n_ids) return MOON_OK;
+    MOON_HIP(ctx, hipSetDevice(ctx->device));
+    // through buffers the session's state does not live in: the ids behind the loop's random numbers, the rows in the
+    // MLP scratch (both are rewritten by whatever call uses them next)
+    uint32_t *ids_tmp = reinterpret_cast<uint32_t *>(m->u_dev);
+    MOON_HIP(ctx, hipMemcpyAsync(ids_tmp, ids, n_ids * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
+    MOON_TRY(launch_embed(ctx, m->wte, ids_tmp, m->mlp, n_ids, m->cfg.dim));
+    MOON_HIP(ctx, hipMemcpyAsync(embeds, m->mlp, n_ids * m->cfg.dim * sizeof(moon_f16), hipMemcpyDeviceToHost, ctx->stream));
     MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
     return MOON_OK;
 }
@@ -648,49 +611,13 @@ static void print_layer_trace(moon_text_model *m) {
     }
 }
 
-// MOON_DECODE_TRACE with the streaming kernel: per layer of the last step, when the workgroups passed the kernel's eight
-// stamps (microseconds after the layer's first workgroup started it; mean and latest over the 256 workgroups)
-static void print_stream_trace(moon_text_model *m) {
-    const Sizes z = sizes(m->cfg);
-    std::vector<long long> t(z.L * size_t(STREAM_GRID) * 8);
-    if (hipMemcpy(t.data(), m->stream_trace, t.size() * sizeof(long long), hipMemcpyDeviceToHost) != hipSuccess) return;
-    const char *names[8] = {"start", "hidden in", "qkv out", "q,k,v in", "attn partial out", "head merged", "partials out", "hidden out"};
-    long long t_first = t[0];
-    for (size_t b = 0; b < STREAM_GRID; b++) t_first = std::min(t_first, t[b * 8]);
-    fprintf(stderr, "[moonhip stream trace] last step, per layer: stamp mean/max us after the layer's first start; layer start after step's first layer start\n");
-    for (size_t l = 0; l < z.L; l++) {
-        const long long *tl = t.data() + l * STREAM_GRID * 8;
-        long long t0 = tl[0];
-        for (size_t b = 0; b < STREAM_GRID; b += 2) t0 = std::min(t0, tl[b * 8]);
-        fprintf(stderr, "  layer %2zu (+%7.1f) attention:", l, (double)(t0 - t_first) * 0.01);
-        for (int i = 1; i < 8; i++) {
-            double sum = 0, mx = 0;
-            for (size_t b = 0; b < STREAM_GRID; b += 2) {
-                const double us = (double)(tl[b * 8 + i] - t0) * 0.01;
-                sum += us;
-                mx = std::max(mx, us);
-            }
-            fprintf(stderr, " %s %.1f/%.1f", names[i], sum / (STREAM_GRID / 2), mx);
-        }
-        fprintf(stderr, " | mlp:");
-        const int mlp_stamps[5] = {0, 1, 2, 3, 6};
-        const char *mlp_names[5] = {"start", "hidden in", "fc1 done", "fc2 done", "partials out"};
-        for (int k = 0; k < 5; k++) {
-            double sum = 0, mx = 0;
-            for (size_t b = 1; b < STREAM_GRID; b += 2) {
-                const double us = (double)(tl[b * 8 + mlp_stamps[k]] - t0) * 0.01;
-                sum += us;
-                mx = std::max(mx, us);
-            }
-            fprintf(stderr, " %s %.1f/%.1f", mlp_names[k], sum / (STREAM_GRID / 2), mx);
-        }
-        fprintf(stderr, "\n");
-    }
-}
-
 // sampling == nullptr: greedy.  Otherwise sampling.sample with u[step] in place of the arg-max (the per-launch kernels only).
+// eos_plus1 != 0: the loop ends when that token (id + 1) comes up; it is not recorded (moondream.zig:341).  *n_out (if set)
+// receives the number of tokens recorded; with an end-of-sequence token set, the host looks at the device's state every
+// EOS_CHUNK steps so that at most that many steps are queued behind the stop.
+constexpr size_t EOS_CHUNK = 8;
 static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, const moon_sampling_config *sampling = nullptr,
-                         const float *u = nullptr) {
+                         const float *u = nullptr, uint32_t eos_plus1 = 0, size_t *n_out = nullptr) {
     moon_ctx *ctx = m->ctx;
     if (!out_ids && n_steps) return moon_fail(ctx, MOON_EINVAL, "text_greedy: null output");
     if (m->cache_invalid) return moon_fail(ctx, MOON_EHIP, "text_greedy: an earlier decode call failed; call moon_text_reset first");
@@ -700,107 +627,11 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
         return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "text_greedy: %zu + %zu tokens > max_seq %zu (SequenceTooLong)", m->cur_len, n_steps, m->cfg.max_seq);
     MOON_HIP(ctx, hipSetDevice(ctx->device));
     if (sampling) MOON_HIP(ctx, hipMemcpyAsync(m->u_dev, u, n_steps * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
-    if (!sampling && m->decode_mode == 4 && m->stream && !m->prof) {
-        const Sizes z = sizes(m->cfg);
-        const StreamLayout lay = stream_layout();
-        if ((uint64_t)m->stream_gen + (uint64_t)n_steps * z.L + 2 > 0xfffffff0ull) { // tags count up for the life of the session
-            MOON_TRY(launch_fill_uniform_u32(ctx, m->stream_sync, lay.words, 0, 0, 1));
-            m->stream_gen = 0;
-        }
-        StreamParams p;
-        p.wte = m->wte; p.ln_w = m->ln_w; p.ln_b = m->ln_b; p.qkv_b = m->qkv_b; p.fc1_b = m->fc1_b;
-        p.fc2_b = m->fc2_b; p.out_b = m->out_b; p.lin_b = m->lin_b; p.lno_w = m->lno_w; p.lno_b = m->lno_b;
-        p.w_base = m->stream_arena; p.w_bytes = m->stream_arena_bytes;
-        p.off_qkv = (uint32_t)((m->qkv_w - m->stream_arena) * sizeof(half_t)); p.off_fc1 = (uint32_t)((m->fc1_w - m->stream_arena) * sizeof(half_t));
-        p.off_fc2t = (uint32_t)((m->fc2_wt - m->stream_arena) * sizeof(half_t)); p.off_outt = (uint32_t)((m->out_wt - m->stream_arena) * sizeof(half_t));
-        p.off_lin = (uint32_t)((m->lin_w - m->stream_arena) * sizeof(half_t));
-        p.cache_k = m->cache_k; p.cache_v = m->cache_v; p.freqs = m->freqs;
-        p.hidden_first = m->hidden + (m->last_n - 1) * z.d; p.hidden_out = m->hidden; p.logits = m->logits;
-        p.hid_t = m->stream_sync + lay.hid; p.qkv_t = m->stream_sync + lay.qkv;
-        p.ap_t = reinterpret_cast<unsigned long long *>(m->stream_sync + lay.ap);
-        p.rp = reinterpret_cast<float *>(m->stream_sync + lay.rp);
-        p.rp_flag = m->stream_sync + lay.rp_flag;
-        p.am_t = reinterpret_cast<unsigned long long *>(m->stream_sync + lay.am);
-        p.error = m->stream_sync + lay.err;
-        p.out_ids = m->ids_dev;
-        p.L = (int)z.L; p.V = (int)z.V; p.rot_dim = (int)m->cfg.rot_dim; p.max_seq = (int)z.S; p.pos0 = (int)m->cur_len; p.n_steps = (int)n_steps;
-        p.eps = m->cfg.ln_eps; p.gen0 = m->stream_gen;
-        p.timeout_ticks = getenv("MOON_STREAM_NOWAIT") ? -1 : 100000000LL; // 1 s of the 100 MHz wall clock
-        p.trace = m->stream_trace;
-        p.debug = getenv("MOON_STREAM_DEBUG") ? atoi(getenv("MOON_STREAM_DEBUG")) : 0;
-        MOON_TRY(launch_decode_stream(ctx, p));
-        m->stream_gen += (uint32_t)(n_steps * z.L);
-        uint32_t error_flag = 0;
-        MOON_HIP(ctx, hipMemcpyAsync(out_ids, m->ids_dev, n_steps * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
-        MOON_HIP(ctx, hipMemcpyAsync(&error_flag, p.error, sizeof(error_flag), hipMemcpyDeviceToHost, ctx->stream));
-        MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
-        if (error_flag != 0) {
-            m->cache_invalid = true;
-            m->last_n = 0;
-            (void)clear_sync_state(m);
-            return moon_fail(ctx, MOON_EHIP, "streaming decode kernel: a wait between workgroups timed out; the session needs moon_text_reset");
-        }
-        if (m->stream_trace) print_stream_trace(m);
-        m->cur_len += n_steps;
-        m->last_n = 1;
-        hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->state_dev, (uint32_t)m->cur_len, 0u);
-        MOON_HIP(ctx, hipGetLastError());
-        return MOON_OK;
-    }
-    if (!sampling && m->decode_mode == 1 && m->groups > 0) {
-        const Sizes z = sizes(m->cfg);
-        DecodeParams p;
-        p.wte = m->wte; p.ln_w = m->ln_w; p.ln_b = m->ln_b; p.qkv_w = m->qkv_w; p.qkv_b = m->qkv_b; p.out_w = m->out_w;
-        p.out_b = m->out_b; p.fc1_w = m->fc1_w; p.fc1_b = m->fc1_b; p.fc2_w = m->fc2_w; p.fc2_b = m->fc2_b; p.lin_w = m->lin_w;
-        p.lin_b = m->lin_b; p.lno_w = m->lno_w; p.lno_b = m->lno_b;
-        p.cache_k = m->cache_k; p.cache_v = m->cache_v; p.freqs = m->freqs;
-        p.hidden = m->hidden; p.hidden_first = m->hidden + (m->last_n - 1) * z.d;
-        p.qkv = m->qkv; p.fc1 = m->fc1; p.attn = m->attn; p.logits = m->logits; p.attn_partial = m->attn_partial;
-        p.amax_val = m->amax_val; p.amax_idx = m->amax_idx; p.out_ids = m->ids_dev; p.sync = m->sync_dev;
-        p.d = (int)z.d; p.ffn = (int)z.ffn; p.H = (int)z.H; p.L = (int)z.L; p.V = (int)z.V; p.rot_dim = (int)m->cfg.rot_dim;
-        p.max_seq = (int)z.S; p.pos0 = (int)m->cur_len; p.n_steps = (int)n_steps; p.eps = m->cfg.ln_eps;
-        // MOON_DECODE_TRACE=1: print where workgroup 0 spent the last step (per phase kind), for tuning
-        const bool trace = getenv("MOON_DECODE_TRACE") != nullptr;
-        const size_t n_ph = 1 + 2 * z.L;
-        p.trace = nullptr;
-        if (trace) {
-            MOON_TRY(moon_grow(ctx, ctx->work[0], n_ph * 4 * sizeof(long long)));
-            p.trace = (long long *)ctx->work[0].ptr;
-        }
-        MOON_TRY(launch_fill_uniform_u32(ctx, m->sync_dev, decode_persistent_sync_words(), 0, 0, 1)); // all zero (a fill kernel, not a memset)
-        MOON_TRY(launch_decode_persistent(ctx, p, m->groups, m->persistent_shmem));
-        uint32_t error_flag = 0;
-        MOON_HIP(ctx, hipMemcpyAsync(out_ids, m->ids_dev, n_steps * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
-        MOON_HIP(ctx, hipMemcpyAsync(&error_flag, m->sync_dev + decode_persistent_error_word(), sizeof(error_flag), hipMemcpyDeviceToHost,
-                                     ctx->stream));
-        MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
-        if (error_flag != 0) return moon_fail(ctx, MOON_EHIP, "persistent decode kernel: device-wide barrier timed out");
-        if (trace) {
-            std::vector<long long> t(n_ph * 4);
-            MOON_HIP(ctx, hipMemcpy(t.data(), p.trace, t.size() * sizeof(long long), hipMemcpyDeviceToHost));
-            const char *names[3] = {"lm_head", "qkv+fc1", "attn+fc2+out"};
-            double sum[3][3] = {};
-            int cnt[3] = {};
-            for (size_t ph = 0; ph < n_ph; ph++) {
-                const int kind = ph == 0 ? 0 : 1 + (int)((ph - 1) & 1);
-                for (int k = 0; k < 3; k++) sum[kind][k] += (double)(t[ph * 4 + k + 1] - t[ph * 4 + k]) * 0.01; // 100 MHz ticks -> us
-                cnt[kind]++;
-            }
-            fprintf(stderr, "[moonhip decode trace] last step, workgroup 0, total %.1f us\n", (double)(t[n_ph * 4 - 1] - t[0]) * 0.01);
-            for (int k = 0; k < 3; k++)
-                fprintf(stderr, "  %-12s x%-3d  before-rows %7.2f us  rows %7.2f us  after-rows %7.2f us (mean)\n", names[k], cnt[k],
-                        sum[k][0] / cnt[k], sum[k][1] / cnt[k], sum[k][2] / cnt[k]);
-        }
-        m->cur_len += n_steps;
-        m->last_n = 1;
-        hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->state_dev, (uint32_t)m->cur_len, 0u);
-        MOON_HIP(ctx, hipGetLastError());
-        return MOON_OK;
-    }
     uint32_t *state = m->state_dev;
-    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, state, (uint32_t)m->cur_len, 0u);
+    hipLaunchKernelGGL(start_loop_kernel, dim3(1), dim3(1), 0, ctx->stream, state, (uint32_t)m->cur_len, eos_plus1);
     MOON_HIP(ctx, hipGetLastError());
-    const int mode = m->decode_mode == 4 ? 0 : m->decode_mode; // sampled decoding and profiled steps take the per-layer kernels
+    if (n_out) *n_out = 0;
+    const int mode = m->decode_mode;
     const bool use_layer = m->whole_layer && mode == 0;
     if (use_layer) { // counters count up for the life of the model: clear them long before 32 bits are used up (192 per launch)
         const Sizes z = sizes(m->cfg);
@@ -857,8 +688,16 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
             }
             p.kinds.clear();
         }
+        if (eos_plus1 && (step + 1) % EOS_CHUNK == 0 && step + 1 < n_steps) { // has the end-of-sequence token come up?
+            uint32_t st[4];
+            MOON_HIP(ctx, hipMemcpyAsync(st, state, sizeof(st), hipMemcpyDeviceToHost, ctx->stream));
+            MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
+            if (st[3]) break;
+        }
     }
     uint32_t front_error = 0;
+    uint32_t final_state[4] = {0, (uint32_t)n_steps, 0, 0};
+    if (eos_plus1) MOON_HIP(ctx, hipMemcpyAsync(final_state, state, sizeof(final_state), hipMemcpyDeviceToHost, ctx->stream));
     MOON_HIP(ctx, hipMemcpyAsync(out_ids, m->ids_dev, n_steps * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
     if (use_layer)
         MOON_HIP(ctx, hipMemcpyAsync(&front_error, m->layer_sync + m->cfg.n_layers * m->layer_sync_words, sizeof(front_error), hipMemcpyDeviceToHost,
@@ -874,8 +713,12 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
         (void)clear_sync_state(m);
         return moon_fail(ctx, MOON_EHIP, "fused decode kernel: a wait between its phases timed out; the session needs moon_text_reset");
     }
-    m->cur_len += n_steps;
-    m->last_n = 1;
+    // every recorded token went through the layers and sits in the cache; after a stop the launches queued behind it have
+    // overwritten the hidden state and the logits, so the session then needs a forward pass before the next loop
+    const size_t recorded = final_state[1];
+    m->cur_len += recorded;
+    m->last_n = final_state[3] ? 0 : 1;
+    if (n_out) *n_out = recorded;
     if (use_layer && m->layer_trace) print_layer_trace(m);
     return MOON_OK;
 }
@@ -903,13 +746,52 @@ extern "C" int moon_text_sample(moon_text_model *m, const moon_sampling_config *
     return greedy_locked(m, n_steps, out_ids, cfg, u);
 }
 
+extern "C" int moon_text_generate(moon_text_model *m, const moon_sampling_config *cfg, const float *u, size_t max_tokens, uint32_t eos_token,
+                                  uint32_t *out_ids, size_t *n_out) {
+    if (!m) return MOON_EINVAL;
+    moon_ctx *ctx = m->ctx;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (!n_out) return moon_fail(ctx, MOON_EINVAL, "text_generate: null count");
+    *n_out = 0;
+    if (eos_token >= m->cfg.vocab) return moon_fail(ctx, MOON_ETOKEN, "text_generate: end-of-sequence id %u >= vocab %zu", eos_token, m->cfg.vocab);
+    // the reference stops at position 2048 (moondream.zig:324) instead of failing: so does this loop
+    if (m->cur_len >= m->cfg.max_seq) return MOON_OK;
+    max_tokens = std::min(max_tokens, m->cfg.max_seq - m->cur_len);
+    const bool greedy = !cfg || cfg->method == MOON_SAMPLE_GREEDY;
+    if (!greedy) {
+        if (!u && max_tokens) return moon_fail(ctx, MOON_EINVAL, "text_generate: null random numbers");
+        if (cfg->method < MOON_SAMPLE_MULTINOMIAL || cfg->method > MOON_SAMPLE_MIN_P)
+            return moon_fail(ctx, MOON_EINVAL, "text_generate: unknown method %d", cfg->method);
+        if (cfg->temperature != 1.0f && !(cfg->temperature > 0.f))
+            return moon_fail(ctx, MOON_ETEMPERATURE, "text_generate: temperature %g (InvalidTemperature)", (double)cfg->temperature);
+        if (cfg->method == MOON_SAMPLE_TOP_K && (!cfg->top_k || std::min(cfg->top_k, m->cfg.vocab) > 1024))
+            return moon_fail(ctx, MOON_EINVAL, "text_generate: top_k %zu (1 to 1024 candidates are sorted on the device)", cfg->top_k);
+    }
+    return greedy_locked(m, max_tokens, out_ids, greedy ? nullptr : cfg, greedy ? nullptr : u, eos_token + 1u, n_out);
+}
+
+extern "C" int moon_text_next_token(moon_text_model *m, const moon_sampling_config *cfg, float u, uint32_t *token) {
+    if (!m) return MOON_EINVAL;
+    moon_ctx *ctx = m->ctx;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (!token) return moon_fail(ctx, MOON_EINVAL, "text_next_token: null output");
+    if (!m->last_n) return moon_fail(ctx, MOON_EINVAL, "text_next_token: no forward pass yet");
+    MOON_HIP(ctx, hipSetDevice(ctx->device));
+    MOON_TRY(lm_head(m, m->last_n - 1));
+    uint32_t *out = m->state_dev + 5; // a word of the loop's state that the loop itself does not use
+    if (!cfg || cfg->method == MOON_SAMPLE_GREEDY) MOON_TRY(launch_argmax(ctx, m->logits, m->cfg.vocab, out));
+    else MOON_TRY(launch_sample(ctx, m->logits, m->cfg.vocab, cfg, u, nullptr, nullptr, nullptr, out));
+    MOON_HIP(ctx, hipMemcpyAsync(token, out, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return MOON_OK;
+}
+
 extern "C" int moon_text_greedy_profile(moon_text_model *m, size_t n_steps, uint32_t *out_ids, float *avg_us, size_t *launches) {
     if (!m) return MOON_EINVAL;
     moon_ctx *ctx = m->ctx;
     std::lock_guard<std::mutex> lock(ctx->mu);
     if (!avg_us || !launches) return moon_fail(ctx, MOON_EINVAL, "text_greedy_profile: null output");
-    if (m->decode_mode == 1 || !m->fused)
-        return moon_fail(ctx, MOON_EINVAL, "text_greedy_profile: only the fused per-layer kernels (decode modes 0 and 2) can be timed per launch");
+    if (!m->fused) return moon_fail(ctx, MOON_EINVAL, "text_greedy_profile: only the fused per-layer kernels can be timed per launch");
     StepProfiler prof;
     m->prof = &prof;
     const int rc = greedy_locked(m, n_steps, out_ids);
@@ -936,22 +818,14 @@ extern "C" int moon_text_debug_raise_wait_error(moon_text_model *m) {
     MOON_HIP(ctx, hipGetLastError());
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->front_sync + z.L * z.H * 32 - 1, 0u, 1u);
     MOON_HIP(ctx, hipGetLastError());
-    if (m->stream) { // the error word sits in a line of its own: {0, 1} to (the unused word before it, the error word)
-        hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->stream_sync + stream_layout().err - 1, 0u, 1u);
-        MOON_HIP(ctx, hipGetLastError());
-    }
     return MOON_OK;
 }
 
 extern "C" int moon_text_set_decode_mode(moon_text_model *m, int mode) {
     if (!m) return MOON_EINVAL;
     std::lock_guard<std::mutex> lock(m->ctx->mu);
-    if (mode < 0 || mode > 4)
-        return moon_fail(m->ctx, MOON_EINVAL,
-                         "decode mode must be 0 (one kernel per layer), 1 (persistent kernel with barriers), 2 (three kernels per layer), 3 (two kernels per "
-                         "layer) or 4 (streaming kernel)");
-    if (mode == 4 && !m->stream) return moon_fail(m->ctx, MOON_EINVAL, "streaming decode kernel unavailable for this configuration or device");
-    if (mode == 1 && m->groups == 0) return moon_fail(m->ctx, MOON_EINVAL, "persistent decode kernel unavailable for this configuration");
+    if (mode != 0 && mode != 2 && mode != 3)
+        return moon_fail(m->ctx, MOON_EINVAL, "decode mode must be 0 (one kernel per layer), 2 (three kernels per layer) or 3 (two kernels per layer)");
     m->decode_mode = mode;
     return MOON_OK;
 }

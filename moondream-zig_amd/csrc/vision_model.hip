@@ -148,15 +148,22 @@ int encode_image_dev(moon_vision_model *m, const half_t *patches, half_t *out) {
     return encode_image_padded(m, out);
 }
 
-// from m->patches_pad[2T, kp] on
-static int encode_image_padded(moon_vision_model *m, half_t *out) {
+// VisionModel.vision_encoder (vision_model.zig:204-271) from m->patches_pad[2T, kp] on: m->enc[2T, dim]
+static int vision_encoder_padded(moon_vision_model *m) {
     moon_ctx *ctx = m->ctx;
     const size_t d = m->cfg.dim, T = m->io_cfg.tokens, Kp = m->kp, R = 2 * T;
     // patch embedding: x = patches . W + b, then += pos_embedding on each crop (:219-229)
     MOON_TRY(launch_gemm(ctx, m->patches_pad, m->pe_w, m->pe_b, m->emb, R, d, Kp, MOON_B_NK, MOON_EPI_BIAS));
     for (size_t img = 0; img < 2; img++) MOON_TRY(launch_add(ctx, m->emb + img * T * d, m->pos, T * d));
     // the encoder blocks and the final LayerNorm on all 2T rows (:231-270)
-    MOON_TRY(encode_dev(m, m->emb, R, m->enc));
+    return encode_dev(m, m->emb, R, m->enc);
+}
+
+// from m->patches_pad[2T, kp] on
+static int encode_image_padded(moon_vision_model *m, half_t *out) {
+    moon_ctx *ctx = m->ctx;
+    const size_t d = m->cfg.dim, T = m->io_cfg.tokens;
+    MOON_TRY(vision_encoder_padded(m));
     // concat(output_0, output_1) along the features (:189-196), then encode_mlp (:366-387)
     for (size_t img = 0; img < 2; img++)
         MOON_HIP(ctx, hipMemcpy2DAsync(m->cat + img * d, 2 * d * sizeof(half_t), m->enc + img * T * d, d * sizeof(half_t), d * sizeof(half_t), T,
@@ -283,6 +290,24 @@ extern "C" int moon_vision_encode_image(moon_vision_model *m, const moon_f16 *pa
     MOON_HIP(ctx, hipMemcpyAsync(ctx->stage[0].ptr, patches, in_bytes, hipMemcpyHostToDevice, ctx->stream));
     MOON_TRY(encode_image_dev(m, (const half_t *)ctx->stage[0].ptr, m->img_out));
     MOON_HIP(ctx, hipMemcpyAsync(out, m->img_out, m->io_cfg.tokens * m->io_cfg.out_dim * sizeof(moon_f16), hipMemcpyDeviceToHost, ctx->stream));
+    MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return MOON_OK;
+}
+
+extern "C" int moon_vision_encoder(moon_vision_model *m, const moon_f16 *patches, moon_f16 *out) {
+    if (!m) return MOON_EINVAL;
+    moon_ctx *ctx = m->ctx;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    if (!m->io) return moon_fail(ctx, MOON_EINVAL, "vision_encoder: no front / back end attached (moon_vision_io_attach)");
+    if (!patches || !out) return moon_fail(ctx, MOON_EINVAL, "vision_encoder: null operand");
+    MOON_HIP(ctx, hipSetDevice(ctx->device));
+    const size_t T = m->io_cfg.tokens, K = m->io_cfg.patch_dim, R = 2 * T, in_bytes = R * K * sizeof(moon_f16);
+    MOON_TRY(moon_grow(ctx, ctx->stage[0], in_bytes));
+    MOON_HIP(ctx, hipMemcpyAsync(ctx->stage[0].ptr, patches, in_bytes, hipMemcpyHostToDevice, ctx->stream));
+    MOON_HIP(ctx, hipMemcpy2DAsync(m->patches_pad, m->kp * sizeof(half_t), ctx->stage[0].ptr, K * sizeof(half_t), K * sizeof(half_t), R,
+                                   hipMemcpyDeviceToDevice, ctx->stream)); // (the pad columns stay zero)
+    MOON_TRY(vision_encoder_padded(m));
+    MOON_HIP(ctx, hipMemcpyAsync(out, m->enc, R * m->cfg.dim * sizeof(moon_f16), hipMemcpyDeviceToHost, ctx->stream));
     MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
     return MOON_OK;
 }

@@ -6,7 +6,7 @@ import ctypes as C
 import numpy as np
 
 from . import _lib as L
-from .context import Context, default_context, ptr
+from .context import InvalidTensorDimension, Context, default_context, ptr
 
 
 def default_config() -> L.TextConfig:
@@ -64,8 +64,7 @@ class TextModel:
         self.ctx.check(self.ctx.lib.moon_text_reset(self.handle))
 
     def set_decode_mode(self, mode: int):
-        """0 (default): one fused kernel per layer; 1: one persistent kernel with device-wide barriers; 2: three kernels per
-        layer; 3: two per layer; 4: the streaming kernel (whole loop in one launch, tagged exchanges between workgroups)."""
+        """0 (default): one fused kernel per layer; 2: three kernels per layer (no waits inside kernels); 3: two per layer."""
         self.ctx.check(self.ctx.lib.moon_text_set_decode_mode(self.handle, mode))
 
     @property
@@ -75,6 +74,26 @@ class TextModel:
     def forward(self, ids):
         ids = np.ascontiguousarray(ids, dtype=np.uint32)
         self.ctx.check(self.ctx.lib.moon_text_forward(self.handle, ptr(ids), ids.size))
+
+    # ---- the reference's own three calls (text_model.zig:106, 139, 325), for a host that keeps its loop
+    def text_encoder(self, ids) -> np.ndarray:
+        """Rows of the embedding table, [n, dim] (text_model.zig:106-137)."""
+        ids = np.ascontiguousarray(ids, dtype=np.uint32).reshape(-1)
+        out = np.empty((ids.size, self.cfg.dim), dtype=np.float16)
+        self.ctx.check(self.ctx.lib.moon_text_embed(self.handle, ptr(ids), ids.size, ptr(out)))
+        return out
+
+    def text_decoder(self, input_embeds) -> np.ndarray:
+        """Appends the rows to the session's cache and returns the decoder's output for them (text_model.zig:139-180)."""
+        e = np.ascontiguousarray(input_embeds, dtype=np.float16)
+        if e.ndim != 2 or e.shape[1] != self.cfg.dim:
+            raise InvalidTensorDimension(f"embeddings of shape {e.shape}")
+        self.ctx.check(self.ctx.lib.moon_text_forward_embeds(self.handle, ptr(e), e.shape[0]))
+        return self.hidden(e.shape[0])
+
+    def lm_head(self) -> np.ndarray:
+        """Logits [1, vocab] of the last row of the latest text_decoder / forward call (text_model.zig:325-345)."""
+        return self.logits().reshape(1, -1)
 
     def hidden(self, n_rows: int) -> np.ndarray:
         out = np.empty((n_rows, self.cfg.dim), dtype=np.float16)
@@ -98,6 +117,25 @@ class TextModel:
         out = np.empty(u.size, dtype=np.uint32)
         self.ctx.check(self.ctx.lib.moon_text_sample(self.handle, C.byref(config), ptr(u), u.size, ptr(out)))
         return out
+
+    def generate(self, max_tokens: int, eos_token: int, config=None, u=None) -> np.ndarray:
+        """The reference's whole generation loop on the device (moondream.zig:323-368): stops at the end-of-sequence token
+        (not part of the result) or at the last cache position.  config None: arg-max."""
+        out = np.empty(max_tokens, dtype=np.uint32)
+        n = C.c_size_t(0)
+        if u is not None:
+            u = np.ascontiguousarray(u, dtype=np.float32).reshape(-1)
+            if u.size < max_tokens:
+                raise ValueError("one random number per step is needed")
+        self.ctx.check(self.ctx.lib.moon_text_generate(self.handle, C.byref(config) if config is not None else None,
+                                                       ptr(u) if u is not None else None, max_tokens, eos_token, ptr(out), C.byref(n)))
+        return out[: n.value].copy()
+
+    def next_token(self, config=None, u: float = 0.0) -> int:
+        """lm_head + sampling.sample on the last position (moondream.zig:333-337); the logits stay on the device."""
+        tok = C.c_uint32(0)
+        self.ctx.check(self.ctx.lib.moon_text_next_token(self.handle, C.byref(config) if config is not None else None, u, C.byref(tok)))
+        return int(tok.value)
 
     PROFILE_KERNELS = ("ln_qkv_fc1", "attention", "out_fc2_residual", "lm_head", "argmax", "bump_pos")
 

@@ -114,6 +114,15 @@ class VisionModel:
         self.ctx.check(self.ctx.lib.moon_vision_encode_image(self.handle, ptr(patches), ptr(out)))
         return out
 
+    def vision_encoder(self, patches) -> np.ndarray:
+        """patches[2 * tokens, patch_dim] -> [2, tokens, dim]: VisionModel.vision_encoder (vision_model.zig:204-271) after its
+        rearrangement into patches: patch embedding, positional embedding, the blocks, the final LayerNorm."""
+        patches = f16(patches)
+        io = getattr(self, "io_cfg", None) or default_io_config()
+        out = np.empty((2, io.tokens, self.cfg.dim), dtype=np.float16)
+        self.ctx.check(self.ctx.lib.moon_vision_encoder(self.handle, ptr(patches), ptr(out)))
+        return out
+
     def encode_image_u8(self, image) -> np.ndarray:
         """VisionModel.encode_image from the resized image on: image[side, side, 3] uint8 -> [tokens, out_dim]."""
         image = np.ascontiguousarray(image)

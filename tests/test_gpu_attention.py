@@ -160,3 +160,32 @@ def test_matrix_core_attention_over_seeded_random_shapes(moon, O, ctx):
         assert err <= TOL, (it, D, H, S, err)
         worst = max(worst, err)
     print(f"\nworst rel-Frobenius over 48 shapes: {worst:.2e}")
+
+
+def test_decode_attention_after_cleanup_starts_from_fresh_counters(moon, O, ctx):
+    """moon_cleanup frees the workspace that holds the per-head counters of the one-launch decode attention
+    (cleanupThreadPool, attention.zig:814).  The next call gets new memory, whatever it holds, at whatever address, and must
+    give the same bits as before: counters that were believed to be still cleared would make the merge run early or never."""
+    H, D, rot, S, pos = 32, 64, 32, 2048, 300
+    qkv = O.fill_normal_f16((3 * H * D,), 0, 10, 1.0)
+    ck = np.zeros((H, S, D), dtype=np.float16)
+    cv = np.zeros((H, S, D), dtype=np.float16)
+    ck[:, :pos] = O.fill_normal_f16((H, pos, D), 0, 11, 1.0)
+    cv[:, :pos] = O.fill_normal_f16((H, pos, D), 0, 12, 1.0)
+    d_qkv, d_tab = ctx.to_device(qkv), ctx.to_device(O.rope_table(rot, S, 10000.0))
+    d_out = ctx.alloc(H * D * 2)
+
+    def step():
+        d_ck, d_cv = ctx.to_device(ck), ctx.to_device(cv)
+        ctx.check(ctx.lib.moon_dev_decode_attention(ctx.handle, d_qkv.ptr, d_ck.ptr, d_cv.ptr, d_tab.ptr, d_out.ptr, H, D, rot, S, pos))
+        ctx.sync()
+        return d_out.to_host((1, H * D))
+
+    first = step()
+    assert np.array_equal(step(), first)  # the counters count on from launch to launch
+    for nbytes in (1 << 16, 1 << 18, 1 << 20, 1 << 22):
+        ctx.cleanup()
+        junk = [ctx.to_device(np.full(nbytes, 0xFF, dtype=np.uint8)) for _ in range(4)]  # what freed memory may come back as
+        del junk
+        assert np.array_equal(step(), first)
+        assert np.array_equal(step(), first)

@@ -202,10 +202,10 @@ def test_vision_encode_image_u8_full_size_front(moon, O, ctx):
 
 
 def _all_modes(dev, ids, n_steps):
-    """(tokens, logits, position) for decode modes 1 (persistent kernel), 0 (one kernel per layer where the device supports
-    it), 2 (three kernels per layer) and 3 (two kernels per layer)."""
+    """(tokens, logits, position) for decode modes 0 (one kernel per layer where the device supports it), 2 (three kernels
+    per layer) and 3 (two kernels per layer)."""
     out = []
-    for mode in (1, 0, 2, 3):
+    for mode in (0, 2, 3):
         dev.reset()
         dev.set_decode_mode(mode)
         dev.forward(ids)
@@ -214,8 +214,8 @@ def _all_modes(dev, ids, n_steps):
     return out
 
 
-def test_persistent_decode_kernel_equals_per_op_kernels_small(moon, O, ctx):
-    """The one-launch greedy loop and the kernel-per-op loop share arithmetic and summation order: same bits."""
+def test_decode_modes_agree_small(moon, O, ctx):
+    """The fused decode kernels of every mode share arithmetic and summation order: same bits."""
     _, dev = _text_pair(moon, O, ctx, SMALL_TEXT)
     ids = O.fill_uniform_u32(20, 0, 54, SMALL_TEXT["vocab"])
     (t1, l1, p1), *others = _all_modes(dev, ids, 40)
@@ -226,7 +226,7 @@ def test_persistent_decode_kernel_equals_per_op_kernels_small(moon, O, ctx):
     dev.close()
 
 
-def test_persistent_decode_kernel_equals_per_op_kernels_full_size(moon, O, ctx):
+def test_decode_modes_agree_full_size(moon, O, ctx):
     """Same check on the real decoder shape (24 x 2048, random-init on the device)."""
     dev = moon.text_model.TextModel(moon.text_model.default_config(), seed=0, std=0.02, ctx=ctx)
     ids = O.fill_uniform_u32(100, 0, 50, 51200)
@@ -273,7 +273,7 @@ def test_sessions_built_from_a_moondream_bin_file(moon, O, ctx, tmp_path):
 
 @pytest.mark.parametrize("case", ["ties", "nan_at_0", "nan_elsewhere", "all_neg_inf", "max_is_last"])
 def test_greedy_argmax_rules_in_every_mode(moon, O, ctx, case):
-    """The greedy loop's arg-max (fused into the LM-head launch in modes 0, 2, 3; inside the persistent kernel in mode 1)
+    """The greedy loop's arg-max (fused into the LM-head launch)
     follows sampling.argmax (sampling.zig:257-273): start from logits[0], move on "greater" only.  The LM-head matrix is
     zero here, so the logits are exactly the crafted bias vector and every step must return the oracle's arg-max of it."""
     cfg = dict(SMALL_TEXT)
@@ -299,7 +299,7 @@ def test_greedy_argmax_rules_in_every_mode(moon, O, ctx, case):
                                        n_heads=cfg["n_heads"], max_seq=cfg["max_seq"])
     dev = moon.text_model.TextModel(mcfg, weights=w, ctx=ctx)
     ids = O.fill_uniform_u32(5, 0, 60, V)
-    for mode in (0, 1, 2, 3):
+    for mode in (0, 2, 3):
         dev.reset()
         dev.set_decode_mode(mode)
         dev.forward(ids)
@@ -331,8 +331,20 @@ def test_session_recovers_after_a_failed_wait(moon, O, ctx):
     dev.forward(ids)
     assert dev.greedy(6).tolist() == want
     assert np.array_equal(dev.logits().view(np.uint16), want_logits.view(np.uint16))
-    # and once more through the two-kernel path and the streaming kernel, whose error words are raised by the same hook
-    for mode in (3, 4):
+    # a single-token forward takes the same fused kernels: it reports the raised word as well, and does not move the position
+    dev.reset()
+    dev.forward(ids)
+    ctx.check(ctx.lib.moon_text_debug_raise_wait_error(dev.handle))
+    with pytest.raises(moon.context.HipError):
+        dev.forward(ids[:1])
+    assert dev.position == 64
+    with pytest.raises(moon.context.HipError):
+        dev.forward(ids[:1])  # refused until reset
+    dev.reset()
+    dev.forward(ids)
+    assert dev.greedy(6).tolist() == want
+    # and once more through the two-kernel path, whose error word is raised by the same hook
+    for mode in (3,):
         dev.reset()
         dev.set_decode_mode(mode)
         dev.forward(ids)
@@ -345,44 +357,160 @@ def test_session_recovers_after_a_failed_wait(moon, O, ctx):
     dev.close()
 
 
-def test_streaming_decode_kernel_against_the_per_layer_kernels(moon, O, ctx):
-    """Decode mode 4 (one launch for the whole greedy loop, weights streamed through LDS rings, workgroups exchanging q/k/v,
-    attention partials, partial sums and the hidden state through tagged words): same ids as the per-layer kernels, hidden
-    state and logits within the end-to-end bound of theirs (out_proj and fc2 are summed in another order), single steps,
-    a run up to the last cache position, and interleaving with forward() calls."""
+def test_generate_stops_at_the_end_of_sequence_token(moon, O, ctx):
+    """moon_text_generate = the loop of moondream.zig:323-368: the tokens before the end-of-sequence token, which is not part
+    of the output (moondream.zig:341); without that token in the stream it runs for max_tokens, or to the end of the cache
+    (moondream.zig:324).  Arg-max and top_k, every decode mode."""
+    ref, dev = _text_pair(moon, O, ctx, SMALL_TEXT)
+    V = SMALL_TEXT["vocab"]
+    ids = O.fill_uniform_u32(20, 0, 57, V)
+    dev.forward(ids)
+    free = dev.greedy(40).tolist()
+    unused = next(t for t in range(V) if t not in free)
+    for mode in (0, 2, 3):
+        dev.set_decode_mode(mode)
+        for stop_at in (0, 1, 7, 8, 9, 23, 39):
+            eos = free[stop_at]
+            first = free.index(eos)  # the token may have come up earlier than where it was picked
+            dev.reset()
+            dev.forward(ids)
+            got = dev.generate(40, eos).tolist()
+            assert got == free[:first], (mode, stop_at)
+            assert dev.position == 20 + first
+            with pytest.raises(moon.InvalidArgument):
+                dev.greedy(1)  # the session needs a forward pass after a stop
+            dev.forward(np.array([eos], dtype=np.uint32))  # ... for example to go on past the token
+            assert dev.position == 20 + first + 1
+        dev.reset()
+        dev.forward(ids)
+        assert dev.generate(40, unused).tolist() == free
+        assert dev.position == 60
+        nxt = dev.greedy(3).tolist()  # without a stop the loop can go on
+        assert nxt == ref_continue(dev, ids, free, 3)
+    dev.set_decode_mode(0)
+    # the end of the cache ends the loop without an error
+    dev.reset()
+    dev.forward(O.fill_uniform_u32(SMALL_TEXT["max_seq"] - 5, 0, 58, V))
+    tail = dev.generate(40, unused)
+    assert tail.size == 5 and dev.position == SMALL_TEXT["max_seq"]
+    assert dev.generate(4, unused).size == 0
+    # sampled: the same tokens as moon_text_sample up to the stop
+    cfg = moon.sampling.sampling_config("top_k", temperature=0.7, top_k=5)
+    u = np.random.default_rng(3).random(30, dtype=np.float32)
+    dev.reset()
+    dev.forward(ids)
+    sampled = dev.sample(cfg, u).tolist()
+    eos = sampled[11]
+    dev.reset()
+    dev.forward(ids)
+    assert dev.generate(30, eos, cfg, u).tolist() == sampled[: sampled.index(eos)]
+    with pytest.raises(moon.TokenIdOutOfBounds):
+        dev.generate(4, V)
+    dev.close()
+
+
+def ref_continue(dev, ids, free, n):
+    """The next n arg-max tokens after ids + free, from a second pass over the same session (what the loop must go on with)."""
+    dev.reset()
+    dev.forward(np.concatenate([ids, np.array(free, dtype=np.uint32)]))
+    return dev.greedy(n).tolist()
+
+
+def test_host_stepped_loop_equals_the_device_loop(moon, O, ctx):
+    """The reference keeps the loop on the host (moondream.zig:323-368): text_decoder on one token, lm_head, sampling.sample,
+    text_encoder.  Through the session that is forward([token]) + next_token() (or logits() and a host-side arg-max) per
+    step: the same 64 ids as moon_text_greedy on the full-size decoder."""
     dev = moon.text_model.TextModel(moon.text_model.default_config(), seed=0, std=0.02, ctx=ctx)
-    ids = O.fill_uniform_u32(50, 0, 50, 51200)
+    ids = O.fill_uniform_u32(768, 0, 50, 51200)
     dev.forward(ids)
-    want = dev.greedy(20).tolist()
-    want_hidden, want_logits = dev.hidden(1).copy(), dev.logits().copy()
+    want = dev.greedy(64).tolist()
     dev.reset()
-    dev.set_decode_mode(4)
     dev.forward(ids)
-    got = dev.greedy(1).tolist() + dev.greedy(1).tolist() + dev.greedy(18).tolist()
+    got = []
+    for step in range(64):
+        tok = dev.next_token()
+        if step % 16 == 0:  # the reference's own form: the logits come back and the host picks
+            assert tok == O.argmax(dev.logits())
+        got.append(tok)
+        dev.forward(np.array([tok], dtype=np.uint32))
     assert got == want
-    assert dev.position == 70
-    assert O.rel_frobenius(dev.hidden(1), want_hidden) <= 4 * TOL
-    assert O.rel_frobenius(dev.logits().reshape(1, -1), want_logits.reshape(1, -1)) <= 4 * TOL
-    # a prompt continuation through forward(), then the loop again: both paths read and extend the same cache
-    more = O.fill_uniform_u32(7, 0, 51, 51200)
-    dev.forward(more)
-    a = dev.greedy(5).tolist()
+    assert dev.position == 768 + 64
+    cfg = moon.sampling.sampling_config("top_k", temperature=0.5, top_k=3)
+    u = np.random.default_rng(1).random(8, dtype=np.float32)
     dev.reset()
-    dev.set_decode_mode(0)
     dev.forward(ids)
-    dev.greedy(20)
-    dev.forward(more)
-    assert dev.greedy(5).tolist() == a
-    # up to the last position of the cache (2048), and not beyond
+    want_s = dev.sample(cfg, u).tolist()
     dev.reset()
-    dev.set_decode_mode(4)
-    dev.forward(O.fill_uniform_u32(2040, 0, 52, 51200))
-    b4 = dev.greedy(8).tolist()
-    assert dev.position == 2048
+    dev.forward(ids)
+    got_s = []
+    for step in range(8):
+        tok = dev.next_token(cfg, float(u[step]))
+        got_s.append(tok)
+        dev.forward(np.array([tok], dtype=np.uint32))
+    assert got_s == want_s
+    dev.close()
+
+
+def test_reference_shaped_calls_of_the_text_session(moon, O, ctx):
+    """TextModel.text_encoder / text_decoder / lm_head as the reference's loop calls them (moondream.zig:323-368), which is
+    what the Zig TextModel drop-in binds: embeddings bit-exact, the decoder on embeddings = the decoder on ids, and the
+    host-kept loop built from the three calls gives the oracle's arg-max ids."""
+    ref, dev = _text_pair(moon, O, ctx, SMALL_TEXT)
+    V = SMALL_TEXT["vocab"]
+    ids = O.fill_uniform_u32(24, 0, 61, V)
+    emb = dev.text_encoder(ids)
+    assert np.array_equal(emb, ref.text_encoder(ids))
+    with pytest.raises(moon.TokenIdOutOfBounds):
+        dev.text_encoder(np.array([3, V], dtype=np.uint32))
+    with pytest.raises(moon.InvalidTensorDimension):
+        dev.text_decoder(emb[:, :-1])
+    cache = ref.new_cache()
+    h_ref = ref.text_decoder(ref.text_encoder(ids), cache)
+    h = dev.text_decoder(emb)
+    assert h.shape == h_ref.shape and O.rel_frobenius(h, h_ref) <= TOL
+    assert dev.position == 24
+    dev.reset()
+    dev.forward(ids)
+    assert np.array_equal(dev.hidden(24), h)  # ids or their embeddings: the same bits
+    lg = dev.lm_head()
+    assert lg.shape == (1, V) and O.rel_frobenius(lg, ref.lm_head(h_ref[-1:])) <= TOL
+    want = dev.greedy(12).tolist()
+    dev.reset()
+    x, got = dev.text_encoder(ids), []
+    for _ in range(12):  # the reference's loop, one row of embeddings per step after the prompt
+        dev.text_decoder(x)
+        tok = O.argmax(dev.lm_head())
+        got.append(tok)
+        x = dev.text_encoder(np.array([tok], dtype=np.uint32))
+    assert got == want
+    # embeddings that are not rows of the table (the image features in front of the prompt, moondream.zig:262-283)
+    feats = O.fill_normal_f16((9, SMALL_TEXT["dim"]), 0, 62, 0.5)
+    cache = ref.new_cache()
+    h_ref = ref.text_decoder(np.concatenate([feats, ref.text_encoder(ids)]), cache)
+    dev.reset()
+    h = dev.text_decoder(np.concatenate([feats, emb]))
+    assert O.rel_frobenius(h, h_ref) <= TOL and dev.position == 33
     with pytest.raises(moon.SequenceTooLong):
-        dev.greedy(1)
-    dev.reset()
-    dev.set_decode_mode(0)
-    dev.forward(O.fill_uniform_u32(2040, 0, 52, 51200))
-    assert dev.greedy(8).tolist() == b4
+        dev.text_decoder(np.zeros((SMALL_TEXT["max_seq"], SMALL_TEXT["dim"]), dtype=np.float16))
+    dev.close()
+
+
+def test_vision_encoder_in_front_of_the_projection(moon, O, ctx):
+    """VisionModel.vision_encoder (vision_model.zig:204-271): patch embedding, positional embedding, the blocks on both crops
+    as one sequence and the final LayerNorm, [2 * tokens, dim]; projecting that on the host gives encode_image's result."""
+    cfg = SMALL_VISION
+    io = dict(patch_dim=20, tokens=27, proj_hidden=96, out_dim=40)
+    w, iw = O.synth_vision_weights(cfg, 0), O.synth_vision_io_weights(cfg, io, 0)
+    ref = O.VisionModel(w, iw, cfg, io)
+    dev = moon.vision_model.VisionModel(moon.vision_model.make_config(**cfg), weights=w, ctx=ctx)
+    patches = O.fill_normal_f16((2 * io["tokens"], io["patch_dim"]), 0, 301, 1.0)
+    with pytest.raises(moon.MoonError):
+        dev.vision_encoder(patches)  # nothing attached yet
+    dev.attach_io(moon.vision_model.make_io_config(**io), weights=iw)
+    got = dev.vision_encoder(patches)
+    want = ref.enc.encode(ref.embed(patches))
+    assert got.shape == (2, io["tokens"], cfg["dim"])  # the reference's shape (vision_model.zig:269)
+    got = got.reshape(2 * io["tokens"], cfg["dim"])
+    assert O.rel_frobenius(got, want) <= TOL
+    assert O.rel_frobenius(dev.encode_image(patches), ref.project(got)) <= TOL
     dev.close()
