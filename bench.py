@@ -12,7 +12,8 @@ Beside it, in the same run:
     attention over the KV cache, fc1 + GELU, out_proj, fc2, residual adds; 100,769,792 bytes of weights and vectors
     plus the layer's K/V prefix per launch, 24 launches per token), timed per launch with HIP event pairs on the
     library's stream inside the same greedy loop, right after the timed steps;
-  * extra: config 1's stand-alone GEMV [1x2048].[2048x8192] (33,591,296 bytes per launch, rotating over 32 weight
+  * extra: the same decoder driven from the host one token per call (the reference's own loop shape) and one decode token
+    through the operator-level C ABI with registered weights; a plain read of one layer launch's bytes; config 1's stand-alone GEMV [1x2048].[2048x8192] (33,591,296 bytes per launch, rotating over 32 weight
     buffers = 1 GiB so the 256 MB last-level cache cannot serve them, with a plain read of the same bytes beside it), the vision fc1/fc2 GEMMs (729x1152x4304, 729x4304x1152), decode / prefill / vision attention and the
     full 27-block vision encoder, each with its own roofline fraction;
   * cpu_baseline: a CPU restatement of the reference's kernels (same blocking and threading as the Zig code; the
@@ -56,6 +57,20 @@ def event_time_us(ctx, launch, iters, warmup=3):
         launch(i)
         total += ctx.timer_stop()
     return total / iters * 1e3
+
+
+def launch_time_us(ctx, launch, iters, warmup=3):
+    """Two figures for one launch: `us`, from ONE event pair around `iters` back-to-back launches (no per-launch event
+    handling inside; the figure a kernel trace's average duration is compared with), and `event_interval_us`, the average of
+    an event pair around every single launch (which adds the command processor's handling of the two events)."""
+    for i in range(warmup):
+        launch(i)
+    ctx.sync()
+    ctx.timer_start()
+    for i in range(iters):
+        launch(i)
+    batch = ctx.timer_stop() / iters * 1e3
+    return batch, event_time_us(ctx, launch, iters, warmup=0)
 
 
 COPY_BYTES = 256 * 2**20
@@ -120,6 +135,7 @@ def bench_decoder(moon, ctx, steps, warmup, decode_mode=None):
                hbm_gbs=(wbytes + kv_bytes) / (dt / steps) / 1e9, first_tokens=toks[:8].tolist(),
                repeats_ms_per_token=[x / steps * 1e3 for x in samples], reported="median of the repeats")
     res["hbm_frac"] = res["hbm_gbs"] / HBM_PEAK_GBS
+    model.bench_ids = ids
     return model, res
 
 
@@ -185,6 +201,137 @@ def profile_decode_kernels(model, us_per_token, mode=None):
     return out
 
 
+def bench_layer_read(ctx, nbytes, iters=96):
+    """The yardstick for the dominant kernel: a kernel that only reads as many bytes as one decoder-layer launch does
+    (weights, vectors and the K/V prefix), rotating over 24 distinct buffers like the 24 layers do, so that the 256 MB
+    last-level cache serves it no better than it serves the decoder."""
+    nbytes = (int(nbytes) + 15) // 16 * 16
+    ring = 24
+    buf = ctx.alloc(ring * nbytes)
+    buf.fill_normal(ring * nbytes // 2, 0, 77, 0.02)
+
+    def read(i):
+        ctx.check(ctx.lib.moon_dev_read(ctx.handle, buf.offset((i % ring) * nbytes), nbytes, None))
+
+    us, us_ev = launch_time_us(ctx, read, iters, warmup=ring)
+    buf.free()
+    return dict(kernel="read16_kernel", bytes=nbytes, ring=ring, us=us, event_interval_us=us_ev, gbs=nbytes / us / 1e3,
+                frac=nbytes / us / 1e3 / HBM_PEAK_GBS)
+
+
+HOST_STEPS = 64
+
+
+def bench_host_stepped(moon, ctx, model, ids):
+    """The reference keeps its generation loop on the host (moondream.zig:323-368).  Two forms of that loop over the
+    device-resident session, HOST_STEPS tokens each from the same prefill, wall clock:
+      session_calls: next_token() (LM head + arg-max on the device, 4 bytes back) and forward([token]) per token;
+      reference_signatures: what the Zig TextModel drop-in does behind text_decoder / lm_head / text_encoder: a row of
+        embeddings up, the hidden row and the row of logits (100 KB) down, arg-max on the host, the next row looked up."""
+    out = {}
+    model.reset()
+    model.forward(ids)
+    ctx.sync()
+    one = np.zeros(1, dtype=np.uint32)
+    for timed in (False, True):
+        n = HOST_STEPS if timed else 4
+        t0 = time.perf_counter()
+        toks = []
+        for _ in range(n):
+            tok = model.next_token()
+            toks.append(tok)
+            one[0] = tok
+            model.forward(one)
+        dt = time.perf_counter() - t0
+    out["session_calls"] = dict(calls_per_token=2, steps=HOST_STEPS, tokens_per_s=HOST_STEPS / dt, ms_per_token=dt / HOST_STEPS * 1e3,
+                                kv_len_start=model.position - HOST_STEPS, first_tokens=toks[:4])
+    model.reset()
+    x = model.text_encoder(ids)
+    model.text_decoder(x)
+    x = model.text_encoder(one)
+    for timed in (False, True):
+        n = HOST_STEPS if timed else 4
+        t0 = time.perf_counter()
+        for _ in range(n):
+            model.text_decoder(x)
+            one[0] = int(np.argmax(model.lm_head()))
+            x = model.text_encoder(one)
+        dt = time.perf_counter() - t0
+    out["reference_signatures"] = dict(calls_per_token=4, steps=HOST_STEPS, tokens_per_s=HOST_STEPS / dt, ms_per_token=dt / HOST_STEPS * 1e3,
+                                       kv_len_start=model.position - HOST_STEPS,
+                                       bytes_per_token=dict(up=2 * D + 4, down=2 * D + 2 * V + 2 * D))
+    return out
+
+
+def bench_op_level_decode(moon, ctx, tokens=3, kv0=PREFILL):
+    """One decode token through the operator-level C ABI (host pointers in, host pointers out, a blocking call per
+    operator) in the reference's call order (text_model.zig:150-172, 182-300, 303-345), all 24 layers' weights registered
+    as resident.  Per layer: layerNorm, Wqkv product + bias, head split, applyRotEmb on q and on k, cache update on the
+    host, singleMaskedSDPA on the host-side cache prefix (6.3 MB up per layer at kv 769), out_proj, fc1 + gelu, fc2, the
+    two adds; then the final layerNorm, the LM head and arg-max.  Every operator is a library call; the head split /
+    merge and the cache update are numpy (the reference does them on the host too).  Wall clock, `tokens` tokens."""
+    ops, hg, att, rope, samp = moon.ops, moon.hgemm_trans, moon.attention, moon.rope, moon.sampling
+    S = 2048
+
+    def synth(shape, stream, std=0.02):
+        n = int(np.prod(shape))
+        buf = ctx.alloc(n * 2)
+        buf.fill_normal(n, 0, stream, std)
+        a = buf.to_host(shape)
+        buf.free()
+        return a
+
+    t0 = time.perf_counter()
+    w = dict(qkv=synth((L, 3 * D, D), 1), out=synth((L, D, D), 2), fc1=synth((L, FFN, D), 3), fc2=synth((L, D, FFN), 4),
+             lin=synth((V, D), 5), wte=synth((V, D), 6))
+    b = dict(qkv=synth((L, 3 * D), 11), out=synth((L, D), 12), fc1=synth((L, FFN), 13), fc2=synth((L, D), 14), lin=synth((V,), 15))
+    ones, zeros = np.ones(D, np.float16), np.zeros(D, np.float16)
+    K = synth((L, H, S, HD), 20, 1.0)
+    Vc = synth((L, H, S, HD), 21, 1.0)
+    table = rope.precompute_freqs_cis(32, S, 10000.0)
+    registered = []
+    for name in ("qkv", "out", "fc1", "fc2"):
+        for l in range(L):
+            ctx.register_weight(w[name][l])
+            registered.append(w[name][l])
+    ctx.register_weight(w["lin"])
+    registered.append(w["lin"])
+    setup_s = time.perf_counter() - t0
+
+    def token(hidden, pos):
+        mask = np.ones((1, 1, pos + 1), dtype=bool)
+        pid = np.array([pos], dtype=np.uint64)
+        for l in range(L):
+            ln = ops.layer_norm(hidden, ones, zeros, ctx=ctx)
+            qkv = ops.broadcast_add_simd(hg.matmul(ln, w["qkv"][l], ctx=ctx), b["qkv"][l], ctx=ctx)
+            q, k, v = (np.ascontiguousarray(qkv[0, i * D:(i + 1) * D].reshape(H, 1, HD)) for i in range(3))
+            q = rope.apply_rot_emb(q, H, HD, table, pid, 32, ctx=ctx)
+            k = rope.apply_rot_emb(k, H, HD, table, pid, 32, ctx=ctx)
+            K[l][:, pos] = k[:, 0]
+            Vc[l][:, pos] = v[:, 0]
+            a = att.single_masked_sdpa(q, K[l][:, :pos + 1], Vc[l][:, :pos + 1], mask, ctx=ctx)
+            a = ops.broadcast_add_simd(hg.matmul(a.reshape(1, D), w["out"][l], ctx=ctx), b["out"][l], ctx=ctx)
+            m = ops.gelu(ops.broadcast_add_simd(hg.matmul(ln, w["fc1"][l], ctx=ctx), b["fc1"][l], ctx=ctx), ctx=ctx)
+            m = ops.broadcast_add_simd(hg.matmul(m, w["fc2"][l], ctx=ctx), b["fc2"][l], ctx=ctx)
+            hidden = ops.add(hidden, ops.add(a, m, ctx=ctx), ctx=ctx)
+        logits = ops.broadcast_add_simd(hg.matmul(ops.layer_norm(hidden, ones, zeros, ctx=ctx), w["lin"], ctx=ctx), b["lin"], ctx=ctx)
+        return samp.argmax(logits, ctx=ctx)
+
+    hidden = w["wte"][7:8].copy()
+    tok = token(hidden, kv0)  # untimed: first use of every kernel and of the staging buffers
+    t0 = time.perf_counter()
+    toks = []
+    for i in range(tokens):
+        tok = token(w["wte"][tok:tok + 1].copy(), kv0 + 1 + i)
+        toks.append(tok)
+    dt = time.perf_counter() - t0
+    for a in registered:
+        ctx.unregister_weight(a)
+    return dict(tokens=tokens, kv_len_start=kv0 + 1, ms_per_token=dt / tokens * 1e3, tokens_per_s=tokens / dt, library_calls_per_token=L * 15 + 4,
+                setup_s=setup_s, tokens_out=toks,
+                note="host pointers and a blocking call per operator; weights resident, activations and the K/V prefix cross the bus every call")
+
+
 def bench_gemv(moon, ctx, iters=256):
     """Config 1: y = f16(f16(x.W^T) + b), x [1,2048], W [8192,2048], rotating over 32 distinct weight buffers (1 GiB) so that
     the 256 MB last-level cache cannot serve them.  Beside it the plain-read kernel on the same buffers: what one launch
@@ -207,14 +354,16 @@ def bench_gemv(moon, ctx, iters=256):
     def read(i):
         ctx.check(ctx.lib.moon_dev_read(ctx.handle, w.offset((i % ring) * N * K * 2), N * K * 2, None))
 
-    us = event_time_us(ctx, launch, iters)
-    us_read = event_time_us(ctx, read, iters)
+    us, us_ev = launch_time_us(ctx, launch, iters)
+    kernel = ctx.last_kernel()
+    us_read, us_read_ev = launch_time_us(ctx, read, iters)
     alg_bytes = N * K * 2 + K * 2 + N * 2 + N * 2
     for buf in (w, x, b, y):
         buf.free()
-    return dict(kernel="gemv_nt_kernel<2,4,BIAS> [1x2048].[2048x8192]^T + bias", us=us, bytes=alg_bytes, gbs=alg_bytes / us / 1e3,
+    return dict(kernel=kernel, shape="[1x2048].[2048x8192]^T + bias", us=us, event_interval_us=us_ev, bytes=alg_bytes, gbs=alg_bytes / us / 1e3,
                 frac=alg_bytes / us / 1e3 / HBM_PEAK_GBS, ring_mib=ring * N * K * 2 / 2**20,
-                plain_read_same_bytes=dict(us=us_read, gbs=N * K * 2 / us_read / 1e3, frac=N * K * 2 / us_read / 1e3 / HBM_PEAK_GBS))
+                plain_read_same_bytes=dict(kernel="read16_kernel", us=us_read, event_interval_us=us_read_ev, gbs=N * K * 2 / us_read / 1e3,
+                                           frac=N * K * 2 / us_read / 1e3 / HBM_PEAK_GBS))
 
 
 def bench_gemm(moon, ctx, M, K, N, iters=50):
@@ -230,11 +379,12 @@ def bench_gemm(moon, ctx, M, K, N, iters=50):
     def launch(i):
         ctx.check(ctx.lib.moon_dev_linear(ctx.handle, a.ptr, M, K, wt.ptr, N, L_.B_NK, b.ptr, L_.EPI_BIAS, c.ptr))
 
-    us = event_time_us(ctx, launch, iters)
+    us, us_ev = launch_time_us(ctx, launch, iters)
+    kernel = ctx.last_kernel()
     flops = 2.0 * M * N * K
     for buf in (a, wt, b, c):
         buf.free()
-    return dict(shape=[M, K, N], us=us, tflops=flops / us / 1e6, frac=flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS)
+    return dict(shape=[M, K, N], kernel=kernel, us=us, event_interval_us=us_ev, tflops=flops / us / 1e6, frac=flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS)
 
 
 def bench_attention(moon, ctx):
@@ -255,9 +405,10 @@ def bench_attention(moon, ctx):
         off = (i % ring) * H * S * HD * 2
         ctx.check(ctx.lib.moon_dev_decode_attention(ctx.handle, qkv.ptr, ck.offset(off), cv.offset(off), tab.ptr, o.ptr, H, HD, 32, S, pos))
 
-    us = event_time_us(ctx, launch, 100)
+    us, us_ev = launch_time_us(ctx, launch, 100)
     nbytes = 2 * H * (pos + 1) * HD * 2 + 2 * 3 * H * HD * 2
-    out["decode_32x64_kv1024"] = dict(us=us, bytes=nbytes, gbs=nbytes / us / 1e3, frac=nbytes / us / 1e3 / HBM_PEAK_GBS)
+    out["decode_32x64_kv1024"] = dict(kernel=ctx.last_kernel(), us=us, event_interval_us=us_ev, bytes=nbytes, gbs=nbytes / us / 1e3,
+                                      frac=nbytes / us / 1e3 / HBM_PEAK_GBS)
     for buf in (ck, cv, qkv, o, tab):
         buf.free()
 
@@ -272,12 +423,13 @@ def bench_attention(moon, ctx):
         def launch(i):
             ctx.check(ctx.lib.moon_dev_sdpa(ctx.handle, q.ptr, k.ptr, v.ptr, oo.ptr, Hh, Lq, Lq, Dd, 0 if causal else -1, None, 0))
 
-        t = event_time_us(ctx, launch, 20)
+        t, t_ev = launch_time_us(ctx, launch, 50)
+        kernel = ctx.last_kernel()
         pairs = Lq * (Lq + 1) // 2 if causal else Lq * Lq
         flops = 4.0 * Hh * Dd * pairs
         for bb in (q, k, v, oo):
             bb.free()
-        return dict(us=t, useful_tflops=flops / t / 1e6, frac=flops / t / 1e6 / MFMA_F16_PEAK_TFLOPS)
+        return dict(kernel=kernel, us=t, event_interval_us=t_ev, useful_tflops=flops / t / 1e6, frac=flops / t / 1e6 / MFMA_F16_PEAK_TFLOPS)
 
     out["prefill_causal_32x768x64"] = sdpa(32, 768, 64, True)
     out["vision_16x729x72"] = sdpa(16, 729, 72, False)
@@ -331,7 +483,7 @@ def bench_vision(moon, ctx, iters=3):
     return res
 
 
-def cpu_baseline(budget_s=20.0):
+def cpu_baseline(budget_s=5.0):
     """Reference-style CPU kernels (oracle/moon_oracle.c: 32-output GEMV chunks, per-head attention, one thread per
     core spawned per call like the Zig code) on a bounded sample: LAYERS_S of the 24 decoder layers plus the LM
     head, a few decode steps at kv_len 769, extrapolated to 24 layers."""
@@ -391,6 +543,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-gemm", action="store_true",
                     help="only the stand-alone GEMM / attention / vision legs, printed as their own JSON line (what a counter run profiles)")
+    ap.add_argument("--only-host-loops", action="store_true", help="only the host-stepped and operator-level decode legs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run 8 plain 256 MiB copies (copy16_kernel) as the known-traffic yardstick for a counter run")
     ap.add_argument("--decode-mode", type=int, default=None,
@@ -413,15 +566,27 @@ def main():
         ctx.close()
         print(json.dumps(out))
         return
+    if args.only_host_loops:
+        model, _ = bench_decoder(moon, ctx, 8, 0)
+        out = {"host_stepped_decode": bench_host_stepped(moon, ctx, model, model.bench_ids)}
+        model.close()
+        out["op_level_decode_registered_weights"] = bench_op_level_decode(moon, ctx)
+        ctx.close()
+        print(json.dumps(out))
+        return
     model, dec = bench_decoder(moon, ctx, args.steps, args.warmup, args.decode_mode)
     kern = profile_decode_kernels(model, dec["ms_per_token"] * 1e3, args.decode_mode)
     sampled = None if args.no_extra else bench_sampled_decode(moon, ctx, model)
+    host_loop = None if args.no_extra else bench_host_stepped(moon, ctx, model, model.bench_ids)
     model.close()
+    yardstick = bench_layer_read(ctx, kern["ln_qkv_fc1"]["bytes"])
     gemv = bench_gemv(moon, ctx)
-    extra = {"decoder": dec, "decode_kernels": kern, "gemv_config1": gemv}
+    extra = {"decoder": dec, "decode_kernels": kern, "plain_read_of_one_layer_launch": yardstick, "gemv_config1": gemv}
     if sampled:
         extra["sampled_decode_top_k"] = sampled
     if not args.no_extra:
+        extra["host_stepped_decode"] = host_loop
+        extra["op_level_decode_registered_weights"] = bench_op_level_decode(moon, ctx)
         extra["gemm_vision_fc1"] = bench_gemm(moon, ctx, 729, 1152, 4304)
         extra["gemm_vision_fc2"] = bench_gemm(moon, ctx, 729, 4304, 1152)
         extra["gemm_vision_fc1_m1458"] = bench_gemm(moon, ctx, 1458, 1152, 4304)
@@ -448,7 +613,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": dom["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"],
                      "traffic": TRAFFIC_BYTES_PER_LAUNCH if "out_fc2_residual" not in kern else None, "kernel": dom_name,
                      "bytes_per_launch": dom["bytes"], "us_per_launch": dom["us"], "event_interval_us": dom["event_interval_us"],
-                     "event_overhead_us": kern["event_overhead_us"], "launches_timed": dom["launches"]},
+                     "event_overhead_us": kern["event_overhead_us"], "launches_timed": dom["launches"],
+                     "plain_read_same_bytes": {"us": yardstick["us"], "gbs": yardstick["gbs"], "frac": yardstick["frac"]}},
         "cpu_baseline": cpu,
         "extra": extra,
     }

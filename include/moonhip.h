@@ -88,6 +88,10 @@ const char *moon_last_error(const moon_ctx *ctx);
  * "dma256", "w114", "w212", "w221"; "" or NULL: chosen by shape, the default).  Every kernel computes the same product to
  * the same rounding points; only the time changes.  The context starts with the value of MOON_GEMM_KERNEL. */
 int moon_set_gemm_kernel(moon_ctx *ctx, const char *name);
+/* Measurement aid without a counterpart in the reference: the name (with its grid and k split) of the kernel that the latest
+ * matrix product, matrix-vector product or attention call on this context dispatched; "" before the first.  The text lives in
+ * the context and changes with the next such call. */
+const char *moon_last_kernel(const moon_ctx *ctx);
 int moon_sync(moon_ctx *ctx);
 /* Releases workspaces. Replaces attention.cleanupThreadPool() (attention.zig:814-818): the
  * reference frees its persistent worker pool there; here it drops cached device buffers. */

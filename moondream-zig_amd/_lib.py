@@ -73,6 +73,7 @@ SIGNATURES = {
     "moon_sync": (_i, [_vp]),
     "moon_cleanup": (None, [_vp]),
     "moon_set_gemm_kernel": (_i, [_vp, C.c_char_p]),
+    "moon_last_kernel": (C.c_char_p, [_vp]),
     "moon_hgemm": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _sz, _vp]),
     "moon_hgemm_trans": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _sz, _vp]),
     "moon_linear": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _i, _vp, _i, _vp]),

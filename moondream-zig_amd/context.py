@@ -115,6 +115,10 @@ class Context:
         """Measurement / test knob: the matrix-product kernel to take where the shape allows it ("" = by shape)."""
         self.check(self.lib.moon_set_gemm_kernel(self.handle, name.encode()))
 
+    def last_kernel(self) -> str:
+        """What the latest product / attention call dispatched (kernel name, grid, k split)."""
+        return self.lib.moon_last_kernel(self.handle).decode()
+
     # ---- resident weights
     def register_weight(self, w: np.ndarray):
         self.check(self.lib.moon_weight_register(self.handle, ptr(w), w.size))

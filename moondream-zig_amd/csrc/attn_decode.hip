@@ -72,6 +72,7 @@ int launch_decode_attention_plain(moon_ctx *ctx, const half_t *q, const half_t *
     MOON_HIP(ctx, hipGetLastError());
     hipLaunchKernelGGL(decode_attn_merge_kernel<64>, dim3((unsigned)H), dim3(64), 0, ctx->stream, partial, out);
     MOON_HIP(ctx, hipGetLastError());
+    MOON_NOTE_KERNEL(ctx, "decode_attn_partial_kernel<64,false> + decode_attn_merge_kernel<64>");
     return MOON_OK;
 }
 
@@ -124,5 +125,6 @@ extern "C" int moon_dev_decode_attention_noalloc(moon_ctx *ctx, const void *qkv,
     MOON_HIP(ctx, hipGetLastError());
     hipLaunchKernelGGL(decode_attn_merge_kernel<64>, dim3((unsigned)n_heads), dim3(64), 0, ctx->stream, partial, (half_t *)out);
     MOON_HIP(ctx, hipGetLastError());
+    MOON_NOTE_KERNEL(ctx, "decode_attn_partial_kernel<64,true> + decode_attn_merge_kernel<64>");
     return MOON_OK;
 }

@@ -78,6 +78,7 @@ int launch_sdpa_generic(moon_ctx *ctx, const half_t *q, const half_t *k, const h
     hipLaunchKernelGGL(sdpa_generic_kernel, dim3((unsigned)((Lq + 3) / 4), (unsigned)H), dim3(256), shmem, ctx->stream, q, k, v, out,
                        (int)H, (int)Lq, (int)Lkv, (int)D, kv_head_stride, causal_pos, mask, mask_stride, out_merged ? 1 : 0, scale);
     MOON_HIP(ctx, hipGetLastError());
+    MOON_NOTE_KERNEL(ctx, "sdpa_generic_kernel");
     return MOON_OK;
 }
 

@@ -370,6 +370,7 @@ int launch_flash(moon_ctx *ctx, const FaArgs &p) {
     }
     hipLaunchKernelGGL(flash_attn_kernel<D>, dim3((unsigned)((p.Lq + FA_Q - 1) / FA_Q), (unsigned)p.H), dim3(256), C::LDS_BYTES, ctx->stream, p);
     MOON_HIP(ctx, hipGetLastError());
+    MOON_NOTE_KERNEL(ctx, "flash_attn_kernel<%d> %d workgroups", D, (int)((p.Lq + FA_Q - 1) / FA_Q) * (int)p.H);
     return MOON_OK;
 }
 

@@ -120,6 +120,8 @@ extern "C" int moon_set_gemm_kernel(moon_ctx *ctx, const char *name) {
     return moon_fail(ctx, MOON_EINVAL, "moon_set_gemm_kernel: unknown kernel \"%s\"", name);
 }
 
+extern "C" const char *moon_last_kernel(const moon_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
+
 extern "C" const char *moon_last_error(const moon_ctx *ctx) { return ctx ? ctx->err.c_str() : g_create_error.c_str(); }
 
 extern "C" int moon_sync(moon_ctx *ctx) {

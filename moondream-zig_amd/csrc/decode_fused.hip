@@ -8,7 +8,9 @@
 // those of gemv.hip / norm.hpp / attn_decode.hpp, so the fused and the unfused paths produce the same bits.
 #include "attn_decode.hpp"
 #include "norm.hpp"
+#include "sample_quick.hpp"
 #include <algorithm>
+#include <cmath>
 #include <cstdlib>
 
 namespace {
@@ -186,7 +188,14 @@ struct LmHeadArgs {
     uint32_t *state;
     uint32_t *out_ids;
     uint32_t bump;
+    // TOPK (the sampled loop with top_k < QUICK_KEYS): partials hold QUICK_WORDS words per workgroup instead of one
+    int top_k;
+    float temperature, scale, inv_t; // scale: 1 / temperature when that is exact, else 0 (as sample_kernel takes it); inv_t: roughly 1 / temperature
+    const float *u_dev;              // u = u_dev[state[1]]
+    uint32_t *decided;               // 1: the token is recorded; 0: sample_kernel has to run
 };
+constexpr int QUICK_WORDS = QUICK_KEYS + 1; // per workgroup: the keys, then (sum bits << 32 | max bits); a bad row travels as a NaN sum
+constexpr int QUICK_MAX_GRID = 1024;        // the merging workgroup's threads take four workgroups' words each, all requested at once
 __device__ __forceinline__ void argmax_merge(float &best, int &idx, float ov, int oi) {
     if (ov > best || (ov == best && oi < idx)) {
         best = ov;
@@ -273,6 +282,171 @@ __global__ __launch_bounds__(256) void decode_lm_head_kernel(LmHeadArgs a) {
         for (int w = 1; w < 4; w++) argmax_merge(best, best_i, s_best[w], s_idx[w]);
         const uint32_t tok = best_i == 0x7fffffff ? 0u : (uint32_t)best_i;
         record_token(a.state, a.out_ids, tok, a.bump);
+    }
+}
+
+// The same launch for the sampled loop with top_k < QUICK_KEYS (the reference CLI's default is top_k 3, moondream.zig:64-65):
+// LayerNorm + LM head, logits to HBM, and per workgroup the QUICK_KEYS largest logits, the maximum and a rough sum of
+// exps; the workgroup that counts in last merges those and decides the token where quick_top_k can prove that it is the
+// reference's (sample_quick.hpp), recording it like the arg-max kernel does and setting *decided; otherwise *decided is 0
+// and sample_kernel, launched behind this kernel either way, evaluates the row in full.
+template <int CH>
+__global__ __launch_bounds__(256) void decode_lm_head_topk_kernel(LmHeadArgs a) {
+    extern __shared__ __attribute__((aligned(16))) half_t s_ln[]; // [d]
+    __shared__ float s_red[16];
+    __shared__ unsigned long long s_keys[4][QUICK_KEYS];
+    __shared__ half_t s_logit[4][64];
+    __shared__ float s_mx[4], s_sum[4];
+    __shared__ unsigned s_bad[4];
+    __shared__ int s_last;
+    constexpr int RG = 4;
+    const LnGemvArgs &p = a.g;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n_waves = gridDim.x * 4, gw = blockIdx.x * 4 + wave;
+    LnInput ln_in;
+    ln_request<true>(ln_in, p.x, p.gamma, p.beta, p.d);
+    int a0, a1;
+    split_rows(p.N1, n_waves, gw, a0, a1);
+    RowGroups<CH, RG> rows;
+    rows.init(p.W1, a0, a1, nullptr, 0, 0, p.d, p.b1);
+    if (rows.total > 0) rows.load(0, lane);
+    layernorm_regs(ln_in, s_ln, p.d, p.eps, s_red);
+    lds_barrier();
+    u32x4 xv[CH];
+    load_x<CH>(xv, s_ln, p.d, lane);
+    const float inv_t = a.inv_t;
+    // Inside the row loop a logit only goes to LDS (the loop is the launch's weight stream: anything more between two row
+    // groups delays the next requests); afterwards lane j takes the wavefront's j-th logit and the wavefront reduces.
+    for (int first = 0; first < rows.total; first += RG) {
+        rows.consume(first, xv, [&](int, int n, float dot, half_t b) {
+            const half_t v = apply_epilogue_v<MOON_EPI_BIAS>(dot, b);
+            if (lane == 0) {
+                p.y1[n] = v;
+                s_logit[wave][n - a0] = v;
+            }
+        });
+        if (first + RG < rows.total) rows.load(first + RG, lane);
+    }
+    QuickTop q; // after the reduction every lane of the wavefront holds the same values
+    quick_init(q);
+    {
+        const bool have = lane < rows.total; // rows.total <= 64 (checked by the launcher)
+        const half_t v = have ? s_logit[wave][lane] : __builtin_bit_cast(half_t, (unsigned short)0xfc00);
+        const unsigned hb = __builtin_bit_cast(unsigned short, v);
+        q.bad = __ballot(have && (hb & 0x7c00u) == 0x7c00u && hb != 0xfc00u) ? 1u : 0u;
+        unsigned long long key = have ? quick_key(v, a0 + lane) : 0ull;
+#pragma unroll
+        for (int r = 0; r < QUICK_KEYS; r++) { // the largest key left, QUICK_KEYS times
+            unsigned long long best = key;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) {
+                const unsigned lo = __shfl_xor((unsigned)best, off, 64), hi = __shfl_xor((unsigned)(best >> 32), off, 64);
+                const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+                best = o > best ? o : best;
+            }
+            q.key[r] = best;
+            if (key == best) key = 0;
+        }
+        if (q.key[0]) {
+            const float mx = (float)quick_key_logit(q.key[0]), f = (float)v;
+            float e = have && f > -INFINITY && mx > -INFINITY ? __expf((f - mx) * inv_t) : 0.f;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) e += __shfl_xor(e, off, 64);
+            q.mx = mx;
+            q.sum = e;
+        }
+    }
+    auto publish = [&]() __attribute__((always_inline)) { // this wavefront's q -> LDS (inlined: q stays in registers)
+        if (lane == 0) {
+#pragma unroll
+            for (int j = 0; j < QUICK_KEYS; j++) s_keys[wave][j] = q.key[j];
+            s_mx[wave] = q.mx;
+            s_sum[wave] = q.sum;
+            s_bad[wave] = q.bad;
+        }
+    };
+    auto gather = [&]() __attribute__((always_inline)) { // thread 0: the other three wavefronts' q merged into its own
+        for (int w = 1; w < 4; w++) {
+            QuickTop o;
+#pragma unroll
+            for (int j = 0; j < QUICK_KEYS; j++) o.key[j] = s_keys[w][j];
+            o.mx = s_mx[w];
+            o.sum = s_sum[w];
+            o.bad = s_bad[w];
+            quick_merge(q, o, inv_t);
+        }
+    };
+    publish();
+    lds_barrier();
+    if (tid == 0) {
+        gather();
+        unsigned long long *mine = a.partials + size_t(blockIdx.x) * QUICK_WORDS;
+#pragma unroll
+        for (int j = 0; j < QUICK_KEYS; j++) __hip_atomic_store(mine + j, q.key[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const float sum_word = q.bad ? __uint_as_float(0x7fc00000u) : q.sum;
+        __hip_atomic_store(mine + QUICK_KEYS, ((unsigned long long)__float_as_uint(sum_word) << 32) | __float_as_uint(q.mx), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the words have reached memory before the workgroup counts in
+        const unsigned leaves = gridDim.x < 32u ? gridDim.x : 32u, leaf = blockIdx.x % leaves;
+        const unsigned members = gridDim.x / leaves + (leaf < gridDim.x % leaves ? 1u : 0u);
+        const uint32_t old = __hip_atomic_fetch_add(a.counter + (1 + leaf) * 32, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = 0;
+        if (old + 1 == a.generation * members) {
+            const uint32_t done = __hip_atomic_fetch_add(a.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = done + 1 == a.generation * leaves ? 1 : 0;
+        }
+    }
+    lds_barrier();
+    if (!s_last) return;
+    quick_init(q);
+    {
+        constexpr int PER = QUICK_MAX_GRID / 256;
+        unsigned long long words[PER][QUICK_WORDS]; // every word is requested before the first is looked at
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int g = tid + i * 256;
+            const unsigned long long *theirs = a.partials + size_t(g < (int)gridDim.x ? g : 0) * QUICK_WORDS;
+#pragma unroll
+            for (int j = 0; j < QUICK_WORDS; j++) words[i][j] = __hip_atomic_load(theirs + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            if (tid + i * 256 >= (int)gridDim.x) continue;
+            QuickTop o;
+#pragma unroll
+            for (int j = 0; j < QUICK_KEYS; j++) o.key[j] = words[i][j];
+            o.mx = __uint_as_float((unsigned)words[i][QUICK_KEYS]);
+            o.sum = __uint_as_float((unsigned)(words[i][QUICK_KEYS] >> 32));
+            o.bad = o.sum != o.sum ? 1u : 0u;
+            if (o.bad) o.sum = 0.f;
+            quick_merge(q, o, inv_t);
+        }
+    }
+    // over the wavefront: a butterfly in which both partners merge the other's q into their own (the keys are distinct
+    // except for the empty key 0, and merging is symmetric: both end with the same q)
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        QuickTop o;
+#pragma unroll
+        for (int j = 0; j < QUICK_KEYS; j++) {
+            const unsigned lo = __shfl_xor((unsigned)q.key[j], off, 64), hi = __shfl_xor((unsigned)(q.key[j] >> 32), off, 64);
+            o.key[j] = ((unsigned long long)hi << 32) | lo;
+        }
+        o.mx = __shfl_xor(q.mx, off, 64);
+        o.sum = __shfl_xor(q.sum, off, 64);
+        o.bad = __shfl_xor(q.bad, off, 64);
+        quick_merge(q, o, inv_t);
+    }
+    lds_barrier();
+    publish();
+    lds_barrier();
+    if (tid == 0) {
+        gather();
+        uint32_t tok = 0;
+        const float u = a.u_dev[a.state[1]];
+        const bool ok = quick_top_k(q, a.top_k, a.temperature, a.scale, u, &tok);
+        if (ok) record_token(a.state, a.out_ids, tok, a.bump);
+        *a.decided = ok ? 1u : 0u;
     }
 }
 
@@ -947,22 +1121,51 @@ int launch_decode_ln_gemv(moon_ctx *ctx, const half_t *x, const uint32_t *token,
 }
 
 // words of the LM head's arg-max exchange: a pair per workgroup (two words each), then the counter lines
-size_t decode_lm_head_words(moon_ctx *ctx) { return size_t(2) * LN_GEMV_GROUPS_PER_CU * (ctx->cu_count > 0 ? ctx->cu_count : 256) + 33 * 32; }
+size_t decode_lm_head_words(moon_ctx *ctx) { return size_t(2 * QUICK_WORDS) * LN_GEMV_GROUPS_PER_CU * (ctx->cu_count > 0 ? ctx->cu_count : 256) + 33 * 32; }
+// (a wavefront of that launch keeps its logits one per lane)
+bool decode_lm_head_top_k_supported(moon_ctx *ctx, size_t top_k, size_t V) {
+    const size_t grid = size_t(LN_GEMV_GROUPS_PER_CU) * (ctx->cu_count > 0 ? ctx->cu_count : 256);
+    return top_k >= 1 && top_k + 1 <= (size_t)QUICK_KEYS && V >= (size_t)QUICK_KEYS && V <= size_t(64) * 4 * grid && grid <= (size_t)QUICK_MAX_GRID;
+}
 int launch_decode_lm_head(moon_ctx *ctx, const half_t *x, const half_t *gamma, const half_t *beta, float eps, size_t d, const half_t *W,
                           const half_t *bias, half_t *logits, size_t V, uint32_t *exchange, uint32_t generation, uint32_t *state,
-                          uint32_t *out_ids, uint32_t bump) {
+                          uint32_t *out_ids, uint32_t bump, const moon_sampling_config *top_k_cfg, const float *u_dev, uint32_t *decided) {
     const unsigned grid = (unsigned)(LN_GEMV_GROUPS_PER_CU * (ctx->cu_count > 0 ? ctx->cu_count : 256));
     if (!V || V > 0x7fffffff) return moon_fail(ctx, MOON_EINVAL, "argmax: empty or oversized tensor");
+    if (top_k_cfg && (!decode_lm_head_top_k_supported(ctx, top_k_cfg->top_k, V) || !u_dev || !decided || !state))
+        return moon_fail(ctx, MOON_EINVAL, "lm head: top_k %zu cannot be decided in the LM-head kernel", top_k_cfg->top_k);
     if ((unsigned long long)generation * grid > 0xffffffffull) return moon_fail(ctx, MOON_EINVAL, "lm head: launch counter out of range");
     LmHeadArgs a;
     a.g = LnGemvArgs{x, nullptr, gamma, beta, W, bias, logits, nullptr, nullptr, nullptr, (int)d, (int)V, 0, eps};
     a.partials = reinterpret_cast<unsigned long long *>(exchange);
-    a.counter = exchange + size_t(2) * grid;
+    a.counter = exchange + size_t(2 * QUICK_WORDS) * grid;
     a.generation = generation;
     a.state = state;
     a.out_ids = out_ids;
     a.bump = bump;
+    a.top_k = 0;
+    a.temperature = a.inv_t = 1.f;
+    a.scale = 0.f;
+    a.u_dev = nullptr;
+    a.decided = nullptr;
     const size_t shmem = d * sizeof(half_t);
+    if (top_k_cfg) {
+        a.top_k = (int)top_k_cfg->top_k;
+        a.temperature = top_k_cfg->temperature;
+        a.inv_t = 1.0f / top_k_cfg->temperature;
+        int exponent = 0; // as launch_sample: dividing by a power of two is a multiplication by its reciprocal, bit for bit
+        a.scale = (std::frexp(top_k_cfg->temperature, &exponent) == 0.5f && exponent > -100 && exponent < 100) ? 1.0f / top_k_cfg->temperature : 0.f;
+        a.u_dev = u_dev;
+        a.decided = decided;
+        switch (pieces(d)) {
+        case 1: hipLaunchKernelGGL((decode_lm_head_topk_kernel<1>), dim3(grid), dim3(256), shmem, ctx->stream, a); break;
+        case 2: hipLaunchKernelGGL((decode_lm_head_topk_kernel<2>), dim3(grid), dim3(256), shmem, ctx->stream, a); break;
+        case 4: hipLaunchKernelGGL((decode_lm_head_topk_kernel<4>), dim3(grid), dim3(256), shmem, ctx->stream, a); break;
+        default: return moon_fail(ctx, MOON_EINVAL_DIM, "fused decode: unsupported dim %zu", d);
+        }
+        MOON_HIP(ctx, hipGetLastError());
+        return MOON_OK;
+    }
     switch (pieces(d)) {
     case 1: hipLaunchKernelGGL((decode_lm_head_kernel<1>), dim3(grid), dim3(256), shmem, ctx->stream, a); break;
     case 2: hipLaunchKernelGGL((decode_lm_head_kernel<2>), dim3(grid), dim3(256), shmem, ctx->stream, a); break;
@@ -998,6 +1201,7 @@ int launch_decode_attention_merged(moon_ctx *ctx, const half_t *qkv, half_t *cac
     hipLaunchKernelGGL(decode_attn_merged_kernel<64>, dim3((unsigned)(H * DEC_SPLITS)), dim3(256), 0, ctx->stream, qkv, cache_k, cache_v, table,
                        partial, out, head_count, count_target, (int)H, (int)rot_dim, (int)max_seq, (int)pos, pos_dev);
     MOON_HIP(ctx, hipGetLastError());
+    MOON_NOTE_KERNEL(ctx, "decode_attn_merged_kernel<64> %d workgroups", (int)(H * DEC_SPLITS));
     return MOON_OK;
 }
 

@@ -893,6 +893,7 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
         const size_t mn = size_t(M) * N;
         hipLaunchKernelGGL(gemm_generic_kernel<EPI>, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, ctx->stream, A, B, bias, resid, C,
                            M, N, K, b_layout == MOON_B_NK ? 1 : 0);
+        MOON_NOTE_KERNEL(ctx, "gemm_generic_kernel");
         MOON_HIP(ctx, hipGetLastError());
         return MOON_OK;
     }
@@ -987,6 +988,7 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
         if (wide == 114) MOON_TRY(go(gemm_nt_wide_kernel<EPI, 1, 1, 4, 64>, WideCfg<1, 1, 4, 64>::LDS_BYTES, set114));
         else if (wide == 212) MOON_TRY(go(gemm_nt_wide_kernel<EPI, 2, 1, 2, 64>, WideCfg<2, 1, 2, 64>::LDS_BYTES, set212));
         else MOON_TRY(go(gemm_nt_wide_kernel<EPI, 2, 2, 1, 32>, WideCfg<2, 2, 1, 32>::LDS_BYTES, set221));
+        MOON_NOTE_KERNEL(ctx, "gemm_nt_wide_kernel<%s> %d workgroups, k split %d", wide == 114 ? "1,1,4,64" : wide == 212 ? "2,1,2,64" : "2,2,1,32", total, splits);
         if (keep_partial) {
             *keep_partial = p.partial;
             *keep_splits = splits;
@@ -1028,6 +1030,7 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
         const dim3 grid2(((total + 7) / 8) * 8);
         if (use192) hipLaunchKernelGGL(gemm_nt_dma192_kernel<EPI>, grid2, dim3(DMA_THREADS), lds_bytes, ctx->stream, p);
         else hipLaunchKernelGGL(gemm_nt_dma256_kernel<EPI>, grid2, dim3(DMA_THREADS), lds_bytes, ctx->stream, p);
+        MOON_NOTE_KERNEL(ctx, "%s %d workgroups", use192 ? "gemm_nt_dma192_kernel" : "gemm_nt_dma256_kernel", total);
         MOON_HIP(ctx, hipGetLastError());
         return MOON_OK;
     }
@@ -1076,6 +1079,8 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     } else {
         hipLaunchKernelGGL(gemm_nt_mfma_kernel<EPI>, dim3(grid), dim3(256), 0, ctx->stream, p);
     }
+    MOON_NOTE_KERNEL(ctx, "%s %d workgroups, k split %d%s", use_dma ? "gemm_nt_dma_kernel" : "gemm_nt_mfma_kernel", total, splits,
+                     splits > 1 ? (ln_ok ? " + splitk_reduce_ln_kernel" : " + splitk_reduce kernel") : "");
     MOON_HIP(ctx, hipGetLastError());
     if (keep_partial) {
         *keep_partial = p.partial;

@@ -102,6 +102,7 @@ int launch_epi(moon_ctx *ctx, const half_t *x, const half_t *W, const half_t *bi
                            ctx->stream, x, W, bias, y, N, K);
     }
     MOON_HIP(ctx, hipGetLastError());
+    MOON_NOTE_KERNEL(ctx, "%s", !vec ? "gemv_nt_generic_kernel" : K >= 4096 ? "gemv_nt_kernel<1,8>" : "gemv_nt_kernel<2,4>");
     return MOON_OK;
 }
 

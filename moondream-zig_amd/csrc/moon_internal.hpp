@@ -32,6 +32,7 @@ struct moon_ctx {
     std::mutex mu;
     std::string err;
     int cu_count = 0;
+    char last_kernel[96] = ""; // moon_last_kernel: what the latest product / attention launch dispatched (set by the launchers)
     char gemm_kernel[8] = ""; // moon_set_gemm_kernel / MOON_GEMM_KERNEL: a product kernel to take where the shape allows it ("": by shape)
     // staging for host-pointer ops: a, b, c, bias/aux, mask
     GrowBuf stage[6];
@@ -52,6 +53,8 @@ struct moon_ctx {
 };
 
 int moon_fail(moon_ctx *ctx, int code, const char *fmt, ...);
+// Notes what a launcher dispatched, for moon_last_kernel (a few dozen nanoseconds per call).
+#define MOON_NOTE_KERNEL(ctx, ...) snprintf((ctx)->last_kernel, sizeof (ctx)->last_kernel, __VA_ARGS__)
 int moon_grow(moon_ctx *ctx, GrowBuf &b, size_t bytes);
 
 #define MOON_HIP(ctx, expr)                                                                          \
@@ -136,8 +139,10 @@ int launch_image_patches(moon_ctx *ctx, const uint8_t *image, half_t *out, size_
 // logits_f32: the row as f32 instead of f16 (then logits is unused).
 // sampling.sample for the methods other than greedy: u, or u_dev[state ? state[1] : 0] when u_dev is set; the token goes to
 // out[0] (if out) and, if state, to state[2] and out_ids[state[1]++], and state[0] += bump_pos (the decode loop's bookkeeping).
+// skip_if: a device word; when it is not 0 as the kernel starts, the kernel does nothing (the step's token is decided already).
 int launch_sample(moon_ctx *ctx, const half_t *logits, size_t n, const moon_sampling_config *cfg, float u, const float *u_dev,
-                  uint32_t *state, uint32_t *out_ids, uint32_t *out, uint32_t bump_pos = 0, const float *logits_f32 = nullptr);
+                  uint32_t *state, uint32_t *out_ids, uint32_t *out, uint32_t bump_pos = 0, const float *logits_f32 = nullptr,
+                  const uint32_t *skip_if = nullptr);
 int launch_embed(moon_ctx *ctx, const half_t *wte, const uint32_t *ids, half_t *out, size_t n_ids, size_t dim);
 int launch_rope_table(moon_ctx *ctx, float *table, size_t rot_dim, size_t end, float theta);
 // x,out [H,S,D]; position_ids on device (u64) or, if null, pos0 + s.

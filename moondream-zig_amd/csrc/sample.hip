@@ -16,6 +16,7 @@
 // the reference's default (top_k 3) the exact path is taken on a few draws in 10^5.
 #pragma clang fp contract(off)
 #include "moon_internal.hpp"
+#include "sample_quick.hpp"
 
 #include <atomic>
 #include <cmath>
@@ -37,6 +38,7 @@ struct SampleArgs {
     uint32_t bump_pos;
     uint32_t *out_ids;
     uint32_t *out;      // when set: out[0] = token
+    const uint32_t *skip_if; // when set and *skip_if != 0: the token of this step is already decided, nothing to do
 };
 
 struct SampleShared {
@@ -54,39 +56,6 @@ struct SampleShared {
     int seq_cross;
     int safe;                    // the quick path's result is provably the exact path's
 };
-
-// exp of the sampling paths: the classic libm expf (k = round(x / ln 2), x - k ln2 in two parts, c = x - x^2 (P1 + x^2 P2),
-// 1 + (x c / (2 - c) - lo + hi), scaled by 2^k) spelled out in separate IEEE f32 operations (this file is compiled with
-// contraction off), because which candidate a draw lands on depends on the last bit of every term: the device and the
-// checker share this definition instead of each trusting its own library's expf.
-__device__ __forceinline__ float sampling_expf(float x) {
-    const float ln2hi = 6.9314575195e-1f, ln2lo = 1.4286067653e-6f, invln2 = 1.4426950216e+0f, P1 = 1.6666625440e-1f, P2 = -2.7667332906e-3f;
-    const unsigned ux = __float_as_uint(x);
-    const int sign = (int)(ux >> 31);
-    const unsigned hx = ux & 0x7fffffffu;
-    if (hx > 0x7f800000u) return x;
-    if (hx >= 0x42b17218u && !sign) return x * 0x1p127f;
-    if (sign && hx >= 0x42cff1b5u) return 0.0f;
-    float hi, lo, xr;
-    int k;
-    if (hx > 0x3eb17218u) {
-        if (hx > 0x3f851592u) k = (int)(invln2 * x + (sign ? -0.5f : 0.5f));
-        else k = 1 - sign - sign;
-        hi = x - (float)k * ln2hi;
-        lo = (float)k * ln2lo;
-        xr = hi - lo;
-    } else if (hx > 0x39000000u) {
-        k = 0;
-        hi = x;
-        lo = 0.0f;
-        xr = x;
-    } else
-        return 1.0f + x;
-    const float xx = xr * xr;
-    const float c = xr - xx * (P1 + xx * P2);
-    const float y = 1.0f + (__fdiv_rn(xr * c, 2.0f - c) - lo + hi);
-    return k == 0 ? y : ldexpf(y, k);
-}
 
 __device__ __forceinline__ float block_max(float v, float *s16) {
 #pragma unroll
@@ -489,6 +458,7 @@ template <int J, int METHOD>
 __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[]; // the staged logits, then SampleShared
     SampleShared &sh = *reinterpret_cast<SampleShared *>(dyn_lds);
+    if (p.skip_if && *p.skip_if) return; // (the same word for every thread: the whole workgroup leaves)
     const int t = threadIdx.x, n = p.n;
     const half_t *__restrict__ logits = p.logits;
     const float *__restrict__ logits_f32 = p.logits_f32;
@@ -696,7 +666,7 @@ hipError_t launch_sample_kernel(hipStream_t stream, const SampleArgs &a) {
 
 // sampling.sample for methods multinomial / top_k / min_p; greedy goes to the arg-max kernels (it ignores the temperature).
 int launch_sample(moon_ctx *ctx, const half_t *logits, size_t n, const moon_sampling_config *cfg, float u, const float *u_dev,
-                  uint32_t *state, uint32_t *out_ids, uint32_t *out, uint32_t bump_pos, const float *logits_f32) {
+                  uint32_t *state, uint32_t *out_ids, uint32_t *out, uint32_t bump_pos, const float *logits_f32, const uint32_t *skip_if) {
     if (!cfg) return moon_fail(ctx, MOON_EINVAL, "sample: null config");
     if (!n || n > 0x3fffffff) return moon_fail(ctx, MOON_EINVAL, "sample: empty or oversized tensor");
     if (cfg->method < MOON_SAMPLE_MULTINOMIAL || cfg->method > MOON_SAMPLE_MIN_P)
@@ -714,7 +684,7 @@ int launch_sample(moon_ctx *ctx, const half_t *logits, size_t n, const moon_samp
     a.temperature = cfg->temperature; a.min_p = cfg->min_p; a.u = u; a.u_dev = u_dev;
     int exponent = 0;
     a.scale = (std::frexp(cfg->temperature, &exponent) == 0.5f && exponent > -100 && exponent < 100) ? 1.0f / cfg->temperature : 0.f;
-    a.state = state; a.out_ids = out_ids; a.out = out; a.bump_pos = bump_pos;
+    a.state = state; a.out_ids = out_ids; a.out = out; a.bump_pos = bump_pos; a.skip_if = skip_if;
     const size_t per_thread = (n + ST - 1) / ST;
     const bool in_registers = !logits_f32 && per_thread <= 64 && (reinterpret_cast<uintptr_t>(logits) & 3) == 0;
     hipError_t e;

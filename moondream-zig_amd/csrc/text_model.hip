@@ -24,7 +24,9 @@ int launch_argmax_record(moon_ctx *ctx, const half_t *logits, size_t n, uint32_t
 size_t decode_lm_head_words(moon_ctx *ctx);
 int launch_decode_lm_head(moon_ctx *ctx, const half_t *x, const half_t *gamma, const half_t *beta, float eps, size_t d, const half_t *W,
                           const half_t *bias, half_t *logits, size_t V, uint32_t *exchange, uint32_t generation, uint32_t *state,
-                          uint32_t *out_ids, uint32_t bump);
+                          uint32_t *out_ids, uint32_t bump, const moon_sampling_config *top_k_cfg = nullptr, const float *u_dev = nullptr,
+                          uint32_t *decided = nullptr);
+bool decode_lm_head_top_k_supported(moon_ctx *ctx, size_t top_k, size_t V);
 bool decode_front_supported(moon_ctx *ctx, size_t d, size_t H, size_t D);
 bool decode_layer_supported(moon_ctx *ctx, size_t d, size_t ffn, size_t H, size_t D);
 size_t decode_layer_sync_words(size_t H);
@@ -651,7 +653,11 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
     }
     size_t row = m->last_n - 1;
     const bool lm_argmax = m->fused && !sampling; // LM head, arg-max and the loop's bookkeeping in one launch
-    if (lm_argmax && (uint64_t(m->lm_launches) + n_steps + 1) * 4096ull > 0x7fffffffull) { // its counter counts up for the life of the model
+    // top_k with a few candidates: the LM-head launch decides the token wherever that is provably the reference's choice and
+    // says so in state[6]; sample_kernel behind it then has nothing to do
+    const bool lm_topk = m->fused && sampling && sampling->method == MOON_SAMPLE_TOP_K && !getenv("MOON_SAMPLE_SEPARATE") &&
+                         decode_lm_head_top_k_supported(ctx, std::min(sampling->top_k, m->cfg.vocab), m->cfg.vocab);
+    if ((lm_argmax || lm_topk) && (uint64_t(m->lm_launches) + n_steps + 1) * 4096ull > 0x7fffffffull) { // its counter counts up for the life of the model
         MOON_TRY(launch_fill_uniform_u32(ctx, m->lm_exchange, decode_lm_head_words(ctx), 0, 0, 1));
         m->lm_launches = 0;
     }
@@ -662,6 +668,16 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
             // token -> state[2], ids[state[1]++]; the position moves on here for every step but the first
             MOON_TRY(launch_decode_lm_head(ctx, m->hidden + row * z.d, m->lno_w, m->lno_b, m->cfg.ln_eps, z.d, m->lin_w, m->lin_b, m->logits, z.V,
                                            m->lm_exchange, ++m->lm_launches, state, m->ids_dev, step > 0 ? 1u : 0u));
+        } else if (lm_topk) {
+            const Sizes z = sizes(m->cfg);
+            {
+                ProfScope scope(m, PROF_LM_HEAD);
+                MOON_TRY(launch_decode_lm_head(ctx, m->hidden + row * z.d, m->lno_w, m->lno_b, m->cfg.ln_eps, z.d, m->lin_w, m->lin_b, m->logits, z.V,
+                                               m->lm_exchange, ++m->lm_launches, state, m->ids_dev, step > 0 ? 1u : 0u, sampling, m->u_dev, state + 6));
+            }
+            ProfScope scope(m, PROF_ARGMAX);
+            MOON_TRY(launch_sample(ctx, m->logits, m->cfg.vocab, sampling, 0.f, m->u_dev, state, m->ids_dev, nullptr, step > 0 ? 1u : 0u, nullptr,
+                                   state + 6));
         } else {
             MOON_TRY(lm_head(m, row));
             ProfScope scope(m, PROF_ARGMAX);

@@ -258,3 +258,97 @@ def test_sample_f32_row(moon, O, ctx):
     greedy = moon.sampling.sampling_config("greedy")
     x[[100, 40000]] = x.max() + 1.0
     assert moon.sampling.sample_f32(x, greedy, 0.0, ctx=ctx) == 100 == moon.sampling.argmax_f32(x, ctx=ctx) == O.sample_f32(x, "greedy", 0.0)
+
+
+def _fixed_logits_model(moon, O, ctx, logits, max_seq=128):
+    """A session whose LM head returns `logits` at every step whatever the hidden state is: a zero matrix and the row as the bias."""
+    cfg = dict(SMALL_TEXT, vocab=logits.size, max_seq=max_seq)
+    w = O.synth_text_weights(cfg, 6)
+    w["linear_w"] = np.zeros_like(w["linear_w"])
+    w["linear_b"] = np.ascontiguousarray(logits, dtype=np.float16)
+    mcfg = moon.text_model.make_config(vocab=cfg["vocab"], dim=cfg["dim"], hidden_dim=cfg["hidden_dim"], n_layers=cfg["n_layers"],
+                                       n_heads=cfg["n_heads"], max_seq=cfg["max_seq"])
+    return moon.text_model.TextModel(mcfg, weights=w, ctx=ctx)
+
+
+def _boundary_us(O, logits, kw, count, seed):
+    """Draws on and next to the candidate boundaries (float32 neighbours of the closed form's cumulative sums), then random ones."""
+    x = logits.astype(np.float64) / kw["temperature"]
+    order = np.lexsort((np.arange(x.size), -x))[: kw["top_k"]]
+    p = np.exp(x[order] - x.max())
+    cum = np.cumsum(p) / p.sum()
+    us = []
+    for c in cum[:-1]:
+        c32 = np.float32(c)
+        us += [c32, np.nextafter(c32, np.float32(0)), np.nextafter(c32, np.float32(1)), np.float32(c * (1 - 3e-6)), np.float32(c * (1 + 3e-6))]
+    us += list(_us(seed, count))
+    return np.array([u for u in us if 0.0 <= u < 1.0], dtype=np.float32)[:count]
+
+
+@pytest.mark.parametrize("kw", [dict(temperature=0.5, top_k=3), dict(temperature=1.0, top_k=1), dict(temperature=0.7, top_k=2),
+                                dict(temperature=1.3, top_k=3)])
+def test_top_k_decided_in_the_lm_head_kernel(moon, O, ctx, kw):
+    """The sampled loop with top_k <= 3 decides the token in the LM-head launch wherever it can prove the choice from the four
+    largest logits, and leaves the rest to sample_kernel.  Rows with the logits fixed (so every step draws from the same
+    row): the oracle's index for every draw, among them draws on the candidate boundaries, ties inside the k, ties across
+    the edge of the k, -inf logits, a row whose exps all but vanish; and the same ids as the loop that runs sample_kernel
+    at every step (MOON_SAMPLE_SEPARATE)."""
+    import os
+    cfg = moon.sampling.sampling_config("top_k", **kw)
+    n = 1000
+    rows = {"normal": _logits(21, n), "steep": _logits(22, n, spread=30.0)}
+    tie_in = _logits(23, n)
+    tie_in[[700, 30]] = tie_in.max() + np.float16(1.0)  # two equal leaders: the lower index first
+    rows["tie_inside"] = tie_in
+    tie_edge = _logits(24, n)
+    top = np.float16(tie_edge.max() + np.float16(2.0))
+    tie_edge[[900, 5, 400, 77, 650]] = [top, top - np.float16(0.5), top - np.float16(1), top - np.float16(1), top - np.float16(1)]
+    rows["tie_across_the_edge"] = tie_edge
+    all_eq = np.full(n, 1.5, dtype=np.float16)
+    rows["all_equal"] = all_eq
+    ninf = _logits(25, n)
+    ninf[::3] = -np.inf
+    rows["minus_inf"] = ninf
+    far = np.full(n, -200.0, dtype=np.float16)
+    far[[10, 20, 30, 40]] = [50.0, -60.0, -61.0, -200.0]
+    rows["vanishing"] = far
+    for name, logits in rows.items():
+        dev = _fixed_logits_model(moon, O, ctx, logits)
+        us = _boundary_us(O, logits, kw, 60, 31)
+        dev.forward(np.array([1, 2, 3], dtype=np.uint32))
+        got = dev.sample(cfg, us).tolist()
+        want = [O.sample(logits, "top_k", float(u), **kw) for u in us]
+        assert got == want, (name, kw)
+        os.environ["MOON_SAMPLE_SEPARATE"] = "1"
+        try:
+            dev.reset()
+            dev.forward(np.array([1, 2, 3], dtype=np.uint32))
+            assert dev.sample(cfg, us).tolist() == got, (name, kw)
+        finally:
+            del os.environ["MOON_SAMPLE_SEPARATE"]
+        dev.close()
+
+
+def test_top_k_in_the_lm_head_kernel_full_size(moon, O, ctx):
+    """The reference CLI's default sampler (top_k 3 at temperature 0.5) on the full-size decoder: the loop that decides in the
+    LM-head launch and the loop that runs sample_kernel at every step give the same 48 ids, and generate() stops both at
+    the same token."""
+    import os
+    dev = moon.text_model.TextModel(moon.text_model.default_config(), seed=0, std=0.02, ctx=ctx)
+    ids = O.fill_uniform_u32(300, 0, 50, 51200)
+    cfg = moon.sampling.sampling_config("top_k", temperature=0.5, top_k=3)
+    us = _us(41, 48)
+    dev.forward(ids)
+    got = dev.sample(cfg, us).tolist()
+    dev.reset()
+    dev.forward(ids)
+    stopped = dev.generate(48, got[20], cfg, us).tolist()
+    assert stopped == got[: got.index(got[20])]
+    os.environ["MOON_SAMPLE_SEPARATE"] = "1"
+    try:
+        dev.reset()
+        dev.forward(ids)
+        assert dev.sample(cfg, us).tolist() == got
+    finally:
+        del os.environ["MOON_SAMPLE_SEPARATE"]
+    dev.close()
