@@ -17,6 +17,7 @@
 #pragma clang fp contract(off)
 #include "moon_internal.hpp"
 #include "sample_quick.hpp"
+#include "seq_sum.hpp"
 
 #include <atomic>
 #include <cmath>
@@ -102,33 +103,6 @@ __device__ __forceinline__ int block_min_int(int v, int *s16) {
 // at most, most of them inside the first chunks.
 // each(f) calls f(i, w_i) for the thread's own indices in ascending order.  On return sh.scan[t] holds the running sum
 // BEFORE chunk t (exact), and the function returns the total.
-struct SeqMap {
-    unsigned c0, c1;
-};
-constexpr unsigned SEQ_BIG = 1u << 24, SEQ_CAP = 1u << 26;
-__device__ __forceinline__ SeqMap seq_compose(SeqMap a, SeqMap b) { // a first, then b
-    SeqMap r;
-    r.c0 = min(a.c0 + ((a.c0 & 1u) ? b.c1 : b.c0), SEQ_CAP);
-    r.c1 = min(a.c1 + (((1u + a.c1) & 1u) ? b.c1 : b.c0), SEQ_CAP);
-    return r;
-}
-// sb: biased exponent of the running sum, 0 when the sum is zero or below the second normal binade (then every non-zero
-// term ends the phase).  Branch-free: this runs for every term in every phase.
-__device__ __forceinline__ SeqMap seq_elem(float w, int sb) {
-    const unsigned bits = __float_as_uint(w);
-    const unsigned ebf = (bits >> 23) & 255u;
-    const unsigned em = (bits & 0x7fffffu) | (ebf ? 0x800000u : 0u); // subnormal: no implicit bit, exponent as for 1
-    const int k = sb - (int)(ebf ? ebf : 1u);                        // w / ulp = em / 2^k
-    const unsigned kc = (unsigned)min(max(k, 1), 25);
-    const unsigned E = em >> kc, frac = em & ((1u << kc) - 1u), half = 1u << (kc - 1u); // em < 2^24: E is 0 from k = 24 on
-    const unsigned up = frac > half ? 1u : 0u, tie = frac == half ? 1u : 0u;
-    SeqMap m{E + up + (tie & E), E + up + (tie & ~E)}; // tie: to the even neighbour, which depends on the parity of S + E
-    const bool zero = (bits << 1) == 0u;
-    const bool big = !zero && (sb == 0 || k <= 0); // no binade to count in, or a term not smaller than the binade itself
-    m.c0 = zero ? 0u : big ? SEQ_BIG : m.c0;
-    m.c1 = zero ? 0u : big ? SEQ_BIG : m.c1;
-    return m;
-}
 template <class Each>
 __device__ __forceinline__ float seq_prefix(Each each, SampleShared &sh) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;

@@ -80,3 +80,21 @@ def test_python_mirror_rejects_bad_ranks_before_calling_c(moon):
         moon.context.f16(np.zeros(4, np.float32))
     assert np.array_equal(moon.hgemm_trans.transpose(np.arange(6, dtype=np.float16).reshape(2, 3)),
                           np.arange(6, dtype=np.float16).reshape(2, 3).T)
+
+
+def test_sequential_sum_maps_equal_the_float_loop():
+    """The sampler evaluates the reference's sequential f32 sums (ops.zig:1585-1592, sampling.zig:139-147, 281-294) by composing
+    per-term integer maps (csrc/seq_sum.hpp).  The host program checks that arithmetic against the plain loop on 20,000 term
+    lists (ties at half an ulp, whole ulps, subnormals, terms rounded away one by one, terms as large as the sum) and the
+    composition's associativity; it needs no GPU."""
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    exe = os.path.join(here, "cxx", "seq_sum_check")
+    src = os.path.join(here, "cxx", "seq_sum_check.cpp")
+    hdr = os.path.join(here, "..", "moondream-zig_amd", "csrc", "seq_sum.hpp")
+    if not os.path.exists(exe) or os.path.getmtime(exe) < max(os.path.getmtime(src), os.path.getmtime(hdr)):
+        subprocess.check_call(["make", "-C", os.path.join(here, "cxx"), "seq_sum_check"])
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    print(r.stdout, r.stderr)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert " 0 failures" in r.stdout

@@ -352,3 +352,28 @@ def test_top_k_in_the_lm_head_kernel_full_size(moon, O, ctx):
     finally:
         del os.environ["MOON_SAMPLE_SEPARATE"]
     dev.close()
+
+
+@pytest.mark.parametrize("method,kw", [("multinomial", dict(temperature=1.0)), ("min_p", dict(temperature=1.2, min_p=0.02))])
+def test_quick_walk_never_differs_from_the_exact_walk_next_to_a_boundary(moon, O, ctx, method, kw):
+    """sample_kernel first takes its sums in whatever order is fast and keeps the answer only if the draw stays (6 m + 32) 2^-24
+    of the total away from the running sums around the chosen candidate (m candidates); otherwise it evaluates the
+    reference's sequential loops bit for bit.  Draws placed on the candidate boundaries of the float64 closed form and at
+    0.5 and 1.5 times that distance on either side: whichever path answers, the index is the oracle's (whose loops are the
+    sequential ones)."""
+    n = 1000
+    logits = _logits(51, n, spread=2.0)
+    x = logits.astype(np.float64) / kw["temperature"]
+    p = np.exp(x - x.max())
+    p /= p.sum()
+    cand = p >= kw["min_p"] * p.max() if method == "min_p" else np.ones(n, bool)
+    m = int(cand.sum())
+    cum = np.cumsum(np.where(cand, p, 0.0))
+    bounds = (cum / cum[-1])[cand][:-1]
+    if bounds.size > 150:
+        bounds = bounds[:: bounds.size // 150]
+    tol = (6.0 * m + 32.0) * 2.0 ** -24
+    us = np.concatenate([bounds + f * tol for f in (-1.5, -0.5, 0.0, 0.5, 1.5)]).astype(np.float32)
+    us = us[(us >= 0) & (us < 1)]
+    assert us.size >= 40, (m, bounds.size)
+    _check(moon, O, ctx, logits, method, us, closed_form=False, **kw)
