@@ -36,8 +36,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense FP16
 
-# HBM bytes per launch of the dominant kernel (decode_layer_kernel) from rocprofv3 counters: FETCH_SIZE 53072.05 KiB x
-# 1.99984 plus WRITE_SIZE 3190.07 KiB x 1.0, the factors being what the same counters read for the 256 MiB copies of
+# HBM bytes per launch of the dominant kernel (decode_layer_kernel) from rocprofv3 counters: FETCH_SIZE 55507.61 KiB x
+# 1.99984 plus WRITE_SIZE 6300.26 KiB x 1.0, the factors being what the same counters read for the 256 MiB copies of
 # --calibrate-copy (profiles/decode_kernels_hbm_traffic_pmc.txt).  A measured constant, not a live reading; it belongs
 # to the default decode mode.
 TRAFFIC_BYTES_PER_LAUNCH = 120_125_663
@@ -561,7 +561,8 @@ def main():
     if args.only_gemm:
         out = {"gemm_vision_fc1": bench_gemm(moon, ctx, 729, 1152, 4304), "gemm_vision_fc2": bench_gemm(moon, ctx, 729, 4304, 1152),
                "gemm_vision_qkv": bench_gemm(moon, ctx, 729, 1152, 3456), "gemm_vision_fc1_m1458": bench_gemm(moon, ctx, 1458, 1152, 4304),
-               "gemm_prefill_fc1": bench_gemm(moon, ctx, 768, 2048, 8192), "attention": bench_attention(moon, ctx),
+               "gemm_prefill_fc1": bench_gemm(moon, ctx, 768, 2048, 8192), "gemm_prefill_fc2": bench_gemm(moon, ctx, 768, 8192, 2048),
+               "gemm_4096": bench_gemm(moon, ctx, 4096, 4096, 4096, iters=20), "attention": bench_attention(moon, ctx),
                "vision_encoder_27_blocks": bench_vision(moon, ctx)}
         ctx.close()
         print(json.dumps(out))
