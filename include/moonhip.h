@@ -289,7 +289,9 @@ int moon_text_greedy(moon_text_model *m, size_t n_steps, uint32_t *out_ids);
 /* The same loop with sampling.sample in place of argmax (moondream.zig:323-368 with a sampling_config other than
  * greedy, moonchat.zig:597): n_steps of lm_head -> sample -> text_encoder([id]) -> text_decoder on the device,
  * logits never leave HBM.  u[n_steps] holds the numbers the reference would draw from its PRNG, one per step
- * (ignored, and may be NULL, for MOON_SAMPLE_GREEDY, which runs moon_text_greedy). */
+ * (ignored, and may be NULL, for MOON_SAMPLE_GREEDY, which runs moon_text_greedy).  With top_k <= 3 the LM-head launch
+ * itself decides the token wherever the four largest logits prove the reference's choice; every other draw, method and
+ * top_k goes through the full evaluation of the row (the kernel behind moon_sample).  The ids are the same either way. */
 int moon_text_sample(moon_text_model *m, const moon_sampling_config *cfg, const float *u, size_t n_steps, uint32_t *out_ids);
 /* The generation loop of moondream.zig:323-368 (moonchat.zig:597-603) on the device: up to max_tokens steps of
  * {lm_head, sampling.sample (cfg == NULL or MOON_SAMPLE_GREEDY: arg-max), text_encoder of the new token, text_decoder},
@@ -420,7 +422,7 @@ int moon_bin_vision_io_weights(const moon_bin *bin, const moon_vision_config *cf
 
 /* ------------------------------------------------------------------------------------------------------------------
  * Environment variables.  None is needed: the defaults are what the tests and the bench run.  They are tuning and
- * diagnostic aids, read once per process (the first call that looks at them fixes the value for every context):
+ * diagnostic aids, read once per process unless noted (the first call that looks at them fixes the value for every context):
  *   MOON_DECODE_TRACE=1            text sessions record per-workgroup time stamps of the last layer launch of a greedy call
  *                                  and print a per-role timeline to stderr (allocated at session creation)
  *   MOON_LAYER_OUT_CHUNK=1|2|4|8|16  decode mode 0: 1 KiB pieces of an fc2 row an output wavefront requests before it waits (default 4)
@@ -429,6 +431,8 @@ int moon_bin_vision_io_weights(const moon_bin *bin, const moon_vision_config *cf
  *   MOON_LAYER_FC1_GROUP=1|2       decode mode 0: fc1 rows a wavefront requests together (default 1)
  *   MOON_GEMM_KERNEL=regs|dma|dma256|w114|w212|w221  forces one of the MFMA product kernels where the shape allows it (default: by shape)
  *   MOON_GEMM_EPILOGUE=direct      the product kernels store their tile without the pass through LDS (default: through LDS)
+ *   MOON_SAMPLE_SEPARATE=1         sampled loops with top_k <= 3: the LM-head launch leaves every token to sample_kernel instead of
+ *                                  deciding it where it provably can (read at every call, so a test can compare the two in one process)
  * Every setting gives the same results, bit for bit; only the time changes. */
 
 #ifdef __cplusplus
