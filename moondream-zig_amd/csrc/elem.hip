@@ -175,6 +175,51 @@ __global__ void qkv_rope_cache_kernel(const half_t *__restrict__ qkv, half_t *__
     ck[co + half] = o_i;
 }
 
+// The same in 16-byte pieces: thread (s, h, g) copies granule g (8 halfs) of v, and of q and k where they are not rotated;
+// granules below rot_dim / 2 rotate themselves against their partners rot_dim / 2 further on and write both.
+// Needs D % 8 == 0, rot_dim % 16 == 0 and 16-byte aligned rows (checked by the launcher).
+__global__ __launch_bounds__(256) void qkv_rope_cache_vec_kernel(const half_t *__restrict__ qkv, half_t *__restrict__ q_out,
+                                                                  half_t *__restrict__ ck, half_t *__restrict__ cv,
+                                                                  const float *__restrict__ table, int S, int H, int D, int rot_dim,
+                                                                  int max_seq, size_t pos0) {
+    const int G = D >> 3;
+    const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= size_t(S) * H * G) return;
+    const int g = int(i % G), h = int((i / G) % H), s = int(i / (size_t(G) * H));
+    const size_t hd = size_t(H) * D;
+    const half_t *row = qkv + size_t(s) * 3 * hd + size_t(h) * D + 8 * g;
+    const size_t qo = (size_t(h) * S + s) * D + 8 * g, co = (size_t(h) * max_seq + pos0 + s) * D + 8 * g;
+    const int half = rot_dim >> 1;
+    *reinterpret_cast<half8_t *>(cv + co) = *reinterpret_cast<const half8_t *>(row + 2 * hd);
+    if (8 * g >= rot_dim) {
+        *reinterpret_cast<half8_t *>(q_out + qo) = *reinterpret_cast<const half8_t *>(row);
+        *reinterpret_cast<half8_t *>(ck + co) = *reinterpret_cast<const half8_t *>(row + hd);
+        return;
+    }
+    if (8 * g >= half) return;
+    const half8_t qr = *reinterpret_cast<const half8_t *>(row), qi = *reinterpret_cast<const half8_t *>(row + half);
+    const half8_t kr = *reinterpret_cast<const half8_t *>(row + hd), ki = *reinterpret_cast<const half8_t *>(row + hd + half);
+    const float4 *t = reinterpret_cast<const float4 *>(table + ((pos0 + s) * half + 8 * g) * 2); // (cos, sin) of 8 consecutive d
+    half8_t oqr, oqi, okr, oki;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const float4 cs = t[e]; // d = 8g + 2e, 8g + 2e + 1
+        half_t a, b;
+        rotate_pair((float)qr[2 * e], (float)qi[2 * e], cs.x, cs.y, a, b);
+        oqr[2 * e] = a; oqi[2 * e] = b;
+        rotate_pair((float)qr[2 * e + 1], (float)qi[2 * e + 1], cs.z, cs.w, a, b);
+        oqr[2 * e + 1] = a; oqi[2 * e + 1] = b;
+        rotate_pair((float)kr[2 * e], (float)ki[2 * e], cs.x, cs.y, a, b);
+        okr[2 * e] = a; oki[2 * e] = b;
+        rotate_pair((float)kr[2 * e + 1], (float)ki[2 * e + 1], cs.z, cs.w, a, b);
+        okr[2 * e + 1] = a; oki[2 * e + 1] = b;
+    }
+    *reinterpret_cast<half8_t *>(q_out + qo) = oqr;
+    *reinterpret_cast<half8_t *>(q_out + qo + half) = oqi;
+    *reinterpret_cast<half8_t *>(ck + co) = okr;
+    *reinterpret_cast<half8_t *>(ck + co + half) = oki;
+}
+
 __global__ void merge_heads_kernel(const half_t *__restrict__ x, half_t *__restrict__ out, int S, int H, int D) {
     const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= size_t(S) * H * D) return;
@@ -302,6 +347,14 @@ int launch_qkv_rope_cache(moon_ctx *ctx, const half_t *qkv, half_t *q_out, half_
                           const float *table, size_t S, size_t H, size_t D, size_t rot_dim, size_t max_seq, size_t pos0) {
     const size_t n = S * H * D;
     if (!n) return MOON_OK;
+    const uintptr_t ptrs = reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(q_out) | reinterpret_cast<uintptr_t>(cache_k) |
+                           reinterpret_cast<uintptr_t>(cache_v) | reinterpret_cast<uintptr_t>(table);
+    if (D % 8 == 0 && rot_dim % 16 == 0 && rot_dim <= D && ptrs % 16 == 0) {
+        hipLaunchKernelGGL(qkv_rope_cache_vec_kernel, dim3(grid_for(n / 8)), dim3(256), 0, ctx->stream, qkv, q_out, cache_k, cache_v, table,
+                           (int)S, (int)H, (int)D, (int)rot_dim, (int)max_seq, pos0);
+        MOON_HIP(ctx, hipGetLastError());
+        return MOON_OK;
+    }
     hipLaunchKernelGGL(qkv_rope_cache_kernel, dim3(grid_for(n)), dim3(256), 0, ctx->stream, qkv, q_out, cache_k, cache_v, table,
                        (int)S, (int)H, (int)D, (int)rot_dim, (int)max_seq, pos0);
     MOON_HIP(ctx, hipGetLastError());
