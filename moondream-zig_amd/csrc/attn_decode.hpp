@@ -4,7 +4,26 @@
 #include "epilogue.hpp"
 
 constexpr int DEC_SPLITS = 8;
-constexpr int DEC_MAX_KEYS = 2048 / DEC_SPLITS; // per split at the reference's kv limit (attention.zig:252)
+constexpr int DEC_MAX_KEYS = (2048 + DEC_SPLITS - 2) / (DEC_SPLITS - 1); // per split at the reference's kv limit (attention.zig:252)
+
+// The key range [j0, j1) of split `split`.  Plain mode: the kv_len keys of the cache in DEC_SPLITS even parts.  Fused mode
+// (the new token's k and v come from the qkv vector): the pos_real cached keys in DEC_SPLITS - 1 even parts, and the new
+// token's own key alone in the last split.  The cached keys need nothing of the new token but q, so only that last split
+// has to wait for its k and v, and it has next to nothing to do once they are there.
+__device__ __forceinline__ void decode_attn_range(int pos_real, bool fused, int split, int &j0, int &j1) {
+    if (!fused) {
+        const int kv_len = pos_real + 1, per = (kv_len + DEC_SPLITS - 1) / DEC_SPLITS;
+        j0 = split * per;
+        j1 = min(kv_len, j0 + per);
+    } else if (split == DEC_SPLITS - 1) {
+        j0 = pos_real;
+        j1 = pos_real + 1;
+    } else {
+        const int per = (pos_real + DEC_SPLITS - 2) / (DEC_SPLITS - 1);
+        j0 = split * per;
+        j1 = min(pos_real, j0 + per);
+    }
+}
 constexpr int DEC_PREFETCH = 4;                 // keys per lane group whose K and V rows are loaded up front
 
 // Merge the DEC_SPLITS partials of one head in a fixed order; returns output element d of that head.
@@ -36,10 +55,9 @@ struct DecodeAttnPrefetch {
 template <int D>
 __device__ __forceinline__ void decode_attn_prefetch(DecodeAttnPrefetch &pf, const half_t *__restrict__ ck, const half_t *__restrict__ cv,
                                                      int max_seq, int pos_real, bool fused, int h, int split) {
-    const int kv_len = pos_real + 1;
     const int pos = fused ? pos_real : -1;
-    const int per = (kv_len + DEC_SPLITS - 1) / DEC_SPLITS;
-    const int j0 = split * per, j1 = min(kv_len, j0 + per);
+    int j0, j1;
+    decode_attn_range(pos_real, fused, split, j0, j1);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 3, e = lane & 7;
     const half_t *kbase = ck + size_t(h) * max_seq * D;
@@ -82,10 +100,9 @@ __device__ __forceinline__ void decode_attn_task(const half_t *__restrict__ qkv,
     __shared__ float sstat[8];
     __shared__ int s_last;
 
-    const int kv_len = pos_real + 1;
     const int pos = FUSED ? pos_real : -1; // in plain mode no key is special
-    const int per = (kv_len + DEC_SPLITS - 1) / DEC_SPLITS;
-    const int j0 = split * per, j1 = min(kv_len, j0 + per);
+    int j0, j1;
+    decode_attn_range(pos_real, FUSED, split, j0, j1);
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int hd = H * D, half = rot_dim >> 1;
     const int g = lane >> 3, e = lane & 7; // key within a group of 8, granule within the key
@@ -101,15 +118,18 @@ __device__ __forceinline__ void decode_attn_task(const half_t *__restrict__ qkv,
         // q stays f16-rounded like the reference's qr tensor; multiplies and adds are separate as in rope.zig
         const int d = t;
         const half_t *q = qkv + h * D, *k = qkv + hd + h * D, *v = qkv + 2 * hd + h * D;
-        sv_new[d] = ld_h<COH>(v + d);
+        // k and v of the new token are read by the split that holds its key alone (a caller may run the other splits
+        // before those rows exist)
+        const bool own = split == DEC_SPLITS - 1;
+        sv_new[d] = own ? ld_h<COH>(v + d) : (half_t)0.0f;
         if (d >= rot_dim) {
             sq[d] = (float)ld_h<COH>(q + d);
-            sk_new[d] = ld_h<COH>(k + d);
+            sk_new[d] = own ? ld_h<COH>(k + d) : (half_t)0.0f;
         } else {
             const int f = d < half ? d : d - half;
             const float c = table[(size_t(pos) * half + f) * 2], sn = table[(size_t(pos) * half + f) * 2 + 1];
-            const float qr = (float)ld_h<COH>(q + f), qi = (float)ld_h<COH>(q + f + half), kr = (float)ld_h<COH>(k + f),
-                        ki = (float)ld_h<COH>(k + f + half);
+            const float qr = (float)ld_h<COH>(q + f), qi = (float)ld_h<COH>(q + f + half);
+            const float kr = own ? (float)ld_h<COH>(k + f) : 0.0f, ki = own ? (float)ld_h<COH>(k + f + half) : 0.0f;
             if (d < half) {
                 sq[d] = (float)(half_t)(qr * c - qi * sn);
                 sk_new[d] = (half_t)(kr * c - ki * sn);

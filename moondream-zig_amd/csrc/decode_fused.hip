@@ -613,8 +613,8 @@ constexpr int LAYER_SYNC_HEADS_DONE = 0;             // line 0: heads merged
 constexpr int LAYER_SYNC_FC1_ROOT = 1;               // line 1: fc1 leaves complete
 constexpr int LAYER_SYNC_FC1_LEAF = 2;               // lines 2..33: fc1 workgroups reported, 32 leaves
 constexpr int LAYER_FC1_LEAVES = 32;
-constexpr int LAYER_SYNC_QKV = 2 + LAYER_FC1_LEAVES; // then one line per head: q, k, v rows written
-inline int layer_sync_words(size_t H) { return (int)(LAYER_SYNC_QKV + H) * LAYER_LINE; }
+constexpr int LAYER_SYNC_QKV = 2 + LAYER_FC1_LEAVES; // then one line per head: q, k, v rows written; then one per head: q rows written
+inline int layer_sync_words(size_t H) { return (int)(LAYER_SYNC_QKV + 2 * H) * LAYER_LINE; }
 
 // thread 0 of the workgroup polls *word until it reaches target; the clock and the error word are looked at once in
 // 64 polls.  Returns (to every thread) whether the wait succeeded.
@@ -714,6 +714,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             const int head = (r0 / 64) % a.H;
             __hip_atomic_fetch_add(a.sync + (LAYER_SYNC_QKV + head) * LAYER_LINE, (uint32_t)(seg_end - r0), __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
+            if (r0 < a.H * 64) // a q row: the splits that do not hold the new token's position wait for these alone
+                __hip_atomic_fetch_add(a.sync + (LAYER_SYNC_QKV + a.H + head) * LAYER_LINE, (uint32_t)(seg_end - r0), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
             r0 = seg_end;
         }
     }
@@ -726,9 +729,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         // and a poll returns in order behind whatever the wavefront has in flight, so it requests its rows afterwards.
         DecodeAttnPrefetch pf;
         if (wave != 0) decode_attn_prefetch<64>(pf, a.ck, a.cv, a.max_seq, pos, true, h, split);
-        if (!wait_reached(a.sync + (LAYER_SYNC_QKV + h) * LAYER_LINE, a.generation * 192u, a.error, &s_flag)) return;
+        // The cached keys need q only; k and v of the new token are one more key, which the last split holds alone
+        // (decode_attn_range).  So that split waits for all of the head's rows, the others for its q rows.
+        if (split == DEC_SPLITS - 1) {
+            if (!wait_reached(a.sync + (LAYER_SYNC_QKV + h) * LAYER_LINE, a.generation * 192u, a.error, &s_flag)) return;
+        } else {
+            if (!wait_reached(a.sync + (LAYER_SYNC_QKV + a.H + h) * LAYER_LINE, a.generation * 64u, a.error, &s_flag)) return;
+        }
         if (wave == 0) decode_attn_prefetch<64>(pf, a.ck, a.cv, a.max_seq, pos, true, h, split);
-        stamp(2); // q, k, v of the head complete
+        stamp(2); // what this split needs of the head's q, k, v is complete
         decode_attn_task<64, true, true>(p.y1, a.ck, a.cv, a.table, a.partial, a.H, a.rot_dim, a.max_seq, pos, h, split, pf, a.head_count,
                                          a.head_target, a.attn_out, a.sync + LAYER_SYNC_HEADS_DONE * LAYER_LINE);
         stamp(3); // task (and possibly the head's merge) done
