@@ -1,7 +1,8 @@
 // C++ host mirror of the reference's operator interface for the FP16 matmul / attention path, over the C ABI in
 // moonhip.h.  The reference is Zig; where no Zig toolchain exists this header plays the part of the .zig shims in
-// ../zig: same namespaces (hgemm, hgemm_trans, attention, rope, ops), same argument meaning, and the reference's
-// error names as exception types.  Header-only; link libmoonhip.so.
+// ../zig: same namespaces (hgemm, hgemm_trans, attention, rope, ops, sampling) and, in namespace model, the reference's
+// TextModel / KVCache / VisionModel over device-resident sessions; same argument meaning, and the reference's error names as
+// exception types.  Header-only; link libmoonhip.so.
 #pragma once
 #include <cstddef>
 #include <cstdint>
@@ -230,5 +231,163 @@ inline Tensor<f16> imagePatches(const Tensor<uint8_t> &image, size_t patch_size,
     return out;
 }
 } // namespace vision
+
+namespace model {
+// The fields of the reference's Weights (weights.zig:16-60) that the two models read, in the moondream.bin layouts.
+struct Weights {
+    Tensor<f16> word_token_embedding, t_ln_w, t_ln_b, t_Wqkv_w, t_Wqkv_b, t_out_proj_w, t_out_proj_bias, t_fc1_w, t_fc1_b, t_fc2_w, t_fc2_b,
+        t_linear_w, t_linear_b, t_ln_out_w, t_ln_out_b;
+    Tensor<f16> v_patch_embedding_linear_w, v_patch_embedding_linear_b, v_pos_embedding, v_Wqkv_w, v_Wqkv_b, v_out_proj_w, v_out_proj_b, v_fc1_w,
+        v_fc1_b, v_fc2_w, v_fc2_b, v_norm1_w, v_norm1_b, v_norm2_w, v_norm2_b, v_norm_out_w, v_norm_out_b, v_proj_fc1_w, v_proj_fc1_b, v_proj_fc2_w,
+        v_proj_fc2_b;
+};
+// config.zig:76-107 (the fields the two models use)
+struct Config {
+    size_t vocab = 51200, dim = 2048, hidden_dim = 8192, n_layers = 24, n_heads = 32, head_dim = 64, seq_len = 2048;
+    size_t img_channels = 3, img_dim = 378, patch_size = 14, vit_dim = 1152, n_vit_layers = 27, n_vit_heads = 16, vit_head_dim = 72,
+           hidden_features = 4304;
+};
+
+class TextModel;
+// KVCache(config) (text_model.zig:349-539): here a handle onto the cache that lives in the TextModel's device session (one live
+// cache per TextModel); reset() empties it.
+class KVCache {
+  public:
+    KVCache() = default;
+    void reset() {
+        if (bound()) moon_text_reset(bound());
+    }
+    size_t getCurrentLen() const { return bound() ? moon_text_position(bound()) : 0; }
+
+  private:
+    friend class TextModel;
+    static moon_text_model *&bound() {
+        static moon_text_model *m = nullptr;
+        return m;
+    }
+};
+
+// TextModel(config) (text_model.zig:22-345) over a device-resident session: text_encoder, text_decoder and lm_head keep the
+// reference's meaning, so the generation loop of moondream.zig:323-368 runs unchanged on top of them.
+class TextModel {
+  public:
+    TextModel(const Config &config, const Weights &w, Context &ctx = Context::global()) : config_(config), ctx_(ctx) {
+        moon_text_config cfg;
+        moon_text_config_default(&cfg);
+        cfg.vocab = config.vocab, cfg.dim = config.dim, cfg.hidden_dim = config.hidden_dim, cfg.n_layers = config.n_layers;
+        cfg.n_heads = config.n_heads, cfg.head_dim = config.head_dim, cfg.rot_dim = config.head_dim / 2, cfg.max_seq = config.seq_len;
+        const moon_text_weights tw{w.word_token_embedding.data.data(), w.t_ln_w.data.data(), w.t_ln_b.data.data(), w.t_Wqkv_w.data.data(),
+                                   w.t_Wqkv_b.data.data(), w.t_out_proj_w.data.data(), w.t_out_proj_bias.data.data(), w.t_fc1_w.data.data(),
+                                   w.t_fc1_b.data.data(), w.t_fc2_w.data.data(), w.t_fc2_b.data.data(), w.t_linear_w.data.data(),
+                                   w.t_linear_b.data.data(), w.t_ln_out_w.data.data(), w.t_ln_out_b.data.data()};
+        ctx_.check(moon_text_model_create(ctx_.get(), &cfg, &tw, &session_));
+        KVCache::bound() = session_;
+    }
+    ~TextModel() {
+        if (KVCache::bound() == session_) KVCache::bound() = nullptr;
+        moon_text_model_destroy(session_);
+    }
+    TextModel(const TextModel &) = delete;
+    TextModel &operator=(const TextModel &) = delete;
+
+    // text_model.zig:106-137
+    Tensor<f16> text_encoder(const Tensor<uint32_t> &input_ids) const {
+        if (input_ids.shape.size() != 1) throw InvalidTensorDimension(MOON_EINVAL_DIM, "InvalidInputShape");
+        Tensor<f16> out({input_ids.shape[0], config_.dim});
+        ctx_.check(moon_text_embed(session_, input_ids.data.data(), input_ids.data.size(), out.data.data()));
+        return out;
+    }
+    // text_model.zig:139-180: the rows are appended at the cache's position (the cache argument is the session's own)
+    struct DecoderResult {
+        Tensor<f16> output;
+        KVCache cache;
+    };
+    DecoderResult text_decoder(const Tensor<f16> &input_embeds, KVCache * /*kv_cache*/) const {
+        if (input_embeds.shape.size() != 2) throw InvalidTensorDimension(MOON_EINVAL_DIM, "InvalidInputShape");
+        const size_t n = input_embeds.shape[0];
+        ctx_.check(moon_text_forward_embeds(session_, input_embeds.data.data(), n));
+        DecoderResult r{Tensor<f16>({n, config_.dim}), KVCache()};
+        ctx_.check(moon_text_hidden(session_, r.output.data.data(), n));
+        return r;
+    }
+    // text_model.zig:325-345: logits of the last row of the latest text_decoder call
+    Tensor<f16> lm_head(const Tensor<f16> &hidden) const {
+        if (hidden.shape.size() != 2) throw InvalidTensorDimension(MOON_EINVAL_DIM, "InvalidInputShape");
+        Tensor<f16> logits({1, config_.vocab});
+        ctx_.check(moon_text_logits(session_, logits.data.data()));
+        return logits;
+    }
+    // lm_head + sampling.sample in one call, the token alone comes back (not in the reference)
+    uint32_t next_token(const sampling::SamplingConfig &config, float u) const {
+        const moon_sampling_config cfg{static_cast<int>(config.method), config.temperature, config.top_k, config.min_p};
+        uint32_t token = 0;
+        ctx_.check(moon_text_next_token(session_, &cfg, u, &token));
+        return token;
+    }
+    moon_text_model *session() const { return session_; }
+
+  private:
+    Config config_;
+    Context &ctx_;
+    moon_text_model *session_ = nullptr;
+};
+
+// VisionModel(config) (vision_model.zig:29-272) from the resized pixels on; decoding and resizing the file stay with the caller.
+class VisionModel {
+  public:
+    VisionModel(const Config &config, const Weights &w, Context &ctx = Context::global()) : config_(config), ctx_(ctx) {
+        moon_vision_config cfg;
+        moon_vision_config_default(&cfg);
+        cfg.dim = config.vit_dim, cfg.hidden_dim = config.hidden_features, cfg.n_layers = config.n_vit_layers, cfg.n_heads = config.n_vit_heads;
+        cfg.head_dim = config.vit_head_dim;
+        const moon_vision_weights vw{w.v_Wqkv_w.data.data(), w.v_Wqkv_b.data.data(), w.v_out_proj_w.data.data(), w.v_out_proj_b.data.data(),
+                                     w.v_fc1_w.data.data(), w.v_fc1_b.data.data(), w.v_fc2_w.data.data(), w.v_fc2_b.data.data(),
+                                     w.v_norm1_w.data.data(), w.v_norm1_b.data.data(), w.v_norm2_w.data.data(), w.v_norm2_b.data.data(),
+                                     w.v_norm_out_w.data.data(), w.v_norm_out_b.data.data()};
+        ctx_.check(moon_vision_model_create(ctx_.get(), &cfg, &vw, &session_));
+        moon_vision_io_config io;
+        moon_vision_io_config_default(&io);
+        tokens_ = (config.img_dim / config.patch_size) * (config.img_dim / config.patch_size);
+        io.patch_dim = config.patch_size * config.patch_size * config.img_channels, io.tokens = tokens_;
+        io.proj_hidden = w.v_proj_fc1_w.shape.at(1), io.out_dim = out_dim_ = w.v_proj_fc2_w.shape.at(1);
+        const moon_vision_io_weights iw{w.v_patch_embedding_linear_w.data.data(), w.v_patch_embedding_linear_b.data.data(),
+                                        w.v_pos_embedding.data.data(), w.v_proj_fc1_w.data.data(), w.v_proj_fc1_b.data.data(),
+                                        w.v_proj_fc2_w.data.data(), w.v_proj_fc2_b.data.data()};
+        const int rc = moon_vision_io_attach(session_, &io, &iw);
+        if (rc != MOON_OK) {
+            moon_vision_model_destroy(session_);
+            session_ = nullptr;
+            ctx_.check(rc);
+        }
+    }
+    ~VisionModel() {
+        if (session_) moon_vision_model_destroy(session_);
+    }
+    VisionModel(const VisionModel &) = delete;
+    VisionModel &operator=(const VisionModel &) = delete;
+
+    // encode_image (vision_model.zig:160-202) from the resized image [img_dim, img_dim, 3] as stbir leaves it
+    Tensor<f16> encode_image(const Tensor<uint8_t> &resized) const {
+        if (resized.shape != std::vector<size_t>{config_.img_dim, config_.img_dim, 3}) throw InvalidTensorDimension(MOON_EINVAL_DIM, "resized image shape");
+        Tensor<f16> out({tokens_, out_dim_});
+        ctx_.check(moon_vision_encode_image_u8(session_, resized.data.data(), out.data.data()));
+        return out;
+    }
+    // vision_encoder (vision_model.zig:204-271) behind rearrangeBCHWtoBTC: patches [2, tokens, patch_dim] -> [2, tokens, vit_dim]
+    Tensor<f16> vision_encoder(const Tensor<f16> &patches) const {
+        if (patches.shape.size() != 3 || patches.shape[0] != 2) throw InvalidTensorDimension(MOON_EINVAL_DIM, "UnexpectedBatchCount");
+        Tensor<f16> out({2, tokens_, config_.vit_dim});
+        ctx_.check(moon_vision_encoder(session_, patches.data.data(), out.data.data()));
+        return out;
+    }
+    moon_vision_model *session() const { return session_; }
+
+  private:
+    Config config_;
+    Context &ctx_;
+    moon_vision_model *session_ = nullptr;
+    size_t tokens_ = 0, out_dim_ = 0;
+};
+} // namespace model
 
 } // namespace moon

@@ -1,5 +1,6 @@
-// Runs the C++ host mirror (hgemm / hgemm_trans / attention / rope entry points and their error behaviour) on the
-// GPU and checks the results against the oracle library loaded beside it.  Exit code 0 = all checks passed.
+// Runs the C++ host mirror (hgemm / hgemm_trans / attention / rope / sampling entry points, the model-level TextModel /
+// KVCache / VisionModel drop-ins and their error behaviour) on the GPU and checks the results against the oracle library
+// loaded beside it, or, for the model-level types, against the session entry points that the Python suite holds to the oracle.  Exit code 0 = all checks passed.
 // Usage: host_mirror_check   (needs libmoonhip.so and libmoon_oracle.so on the link path; see test_gpu_cxx_mirror.py)
 #include <cmath>
 #include <cstdio>
@@ -146,6 +147,98 @@ int main() {
             moon::vision::imagePatches(odd, 2);
             expect(false, "5 rows of 2-pixel patches must throw");
         } catch (const moon::InvalidTensorDimension &) { expect(true, "InvalidPatchSize"); }
+    }
+    // model.TextModel / KVCache: the reference's loop (moondream.zig:323-368) over text_decoder / lm_head / text_encoder gives the
+    // ids of the device loop on the same session; text_encoder returns the table's rows
+    {
+        moon::model::Config cfg;
+        cfg.vocab = 512, cfg.dim = 128, cfg.hidden_dim = 256, cfg.n_layers = 2, cfg.n_heads = 2, cfg.head_dim = 64, cfg.seq_len = 64;
+        moon::model::Weights w;
+        const size_t L = cfg.n_layers, d = cfg.dim, f = cfg.hidden_dim, V = cfg.vocab;
+        auto mk = [](Tensor<f16> &t, std::initializer_list<size_t> shape, float scale) {
+            t = Tensor<f16>(shape);
+            fill(t, scale);
+        };
+        mk(w.word_token_embedding, {V, d}, 0.5f), mk(w.t_ln_w, {L, d}, 1.0f), mk(w.t_ln_b, {L, d}, 0.1f);
+        mk(w.t_Wqkv_w, {L, 3 * d, d}, 0.08f), mk(w.t_Wqkv_b, {L, 3 * d}, 0.05f), mk(w.t_out_proj_w, {L, d, d}, 0.08f);
+        mk(w.t_out_proj_bias, {L, d}, 0.05f), mk(w.t_fc1_w, {L, f, d}, 0.08f), mk(w.t_fc1_b, {L, f}, 0.05f), mk(w.t_fc2_w, {L, d, f}, 0.08f);
+        mk(w.t_fc2_b, {L, d}, 0.05f), mk(w.t_linear_w, {V, d}, 0.08f), mk(w.t_linear_b, {V}, 0.05f), mk(w.t_ln_out_w, {d}, 1.0f);
+        mk(w.t_ln_out_b, {d}, 0.1f);
+        moon::model::TextModel tm(cfg, w);
+        Tensor<uint32_t> ids({6});
+        const uint32_t prompt[6] = {3, 500, 17, 42, 255, 8};
+        for (size_t i = 0; i < 6; i++) ids.data[i] = prompt[i];
+        auto emb = tm.text_encoder(ids);
+        bool rows = emb.shape == std::vector<size_t>{6, d};
+        for (size_t i = 0; i < 6 && rows; i++)
+            rows = std::memcmp(&emb.data[i * d], &w.word_token_embedding.data[prompt[i] * d], d * sizeof(f16)) == 0;
+        expect(rows, "model.TextModel.text_encoder rows");
+        moon::model::KVCache cache;
+        std::vector<uint32_t> host_ids;
+        auto r = tm.text_decoder(emb, &cache);
+        for (int step = 0; step < 5; step++) {
+            auto logits = tm.lm_head(r.output);
+            const uint32_t tok = (uint32_t)moon::sampling::argmax(logits);
+            host_ids.push_back(tok);
+            Tensor<uint32_t> one({1});
+            one.data[0] = tok;
+            r = tm.text_decoder(tm.text_encoder(one), &cache);
+        }
+        expect(cache.getCurrentLen() == 11, "model.KVCache position after the loop", (double)cache.getCurrentLen());
+        cache.reset();
+        expect(cache.getCurrentLen() == 0, "model.KVCache.reset");
+        uint32_t dev_ids[5] = {0, 0, 0, 0, 0};
+        bool ok = moon_text_forward(tm.session(), prompt, 6) == MOON_OK && moon_text_greedy(tm.session(), 5, dev_ids) == MOON_OK;
+        for (int i = 0; i < 5; i++) ok = ok && dev_ids[i] == host_ids[i];
+        expect(ok, "model.TextModel host loop == device loop");
+        cache.reset();
+        moon_text_forward(tm.session(), prompt, 6);
+        moon::sampling::SamplingConfig greedy{moon::sampling::SamplingMethod::greedy};
+        expect(tm.next_token(greedy, 0.0f) == host_ids[0], "model.TextModel.next_token");
+        try {
+            Tensor<uint32_t> bad({1});
+            bad.data[0] = (uint32_t)V;
+            tm.text_encoder(bad);
+            expect(false, "token id == vocab must throw");
+        } catch (const moon::TokenIdOutOfBounds &) { expect(true, "TokenIdOutOfBounds"); }
+    }
+    // model.VisionModel: encode_image from the resized pixels = imagePatches + the session's encode_image on the patches
+    {
+        moon::model::Config cfg;
+        cfg.img_dim = 8, cfg.patch_size = 2, cfg.vit_dim = 128, cfg.n_vit_layers = 2, cfg.n_vit_heads = 2, cfg.vit_head_dim = 64;
+        cfg.hidden_features = 256;
+        const size_t L = cfg.n_vit_layers, d = cfg.vit_dim, f = cfg.hidden_features, T = 16, pd = 12, ph = 96, od = 40;
+        moon::model::Weights w;
+        auto mk = [](Tensor<f16> &t, std::initializer_list<size_t> shape, float scale) {
+            t = Tensor<f16>(shape);
+            fill(t, scale);
+        };
+        mk(w.v_patch_embedding_linear_w, {pd, d}, 0.2f), mk(w.v_patch_embedding_linear_b, {d}, 0.05f), mk(w.v_pos_embedding, {1, T, d}, 0.1f);
+        mk(w.v_Wqkv_w, {L, d, 3 * d}, 0.08f), mk(w.v_Wqkv_b, {L, 3 * d}, 0.05f), mk(w.v_out_proj_w, {L, d, d}, 0.08f), mk(w.v_out_proj_b, {L, d}, 0.05f);
+        mk(w.v_fc1_w, {L, d, f}, 0.08f), mk(w.v_fc1_b, {L, f}, 0.05f), mk(w.v_fc2_w, {L, f, d}, 0.08f), mk(w.v_fc2_b, {L, d}, 0.05f);
+        mk(w.v_norm1_w, {L, d}, 1.0f), mk(w.v_norm1_b, {L, d}, 0.1f), mk(w.v_norm2_w, {L, d}, 1.0f), mk(w.v_norm2_b, {L, d}, 0.1f);
+        mk(w.v_norm_out_w, {d}, 1.0f), mk(w.v_norm_out_b, {d}, 0.1f), mk(w.v_proj_fc1_w, {2 * d, ph}, 0.08f), mk(w.v_proj_fc1_b, {ph}, 0.05f);
+        mk(w.v_proj_fc2_w, {ph, od}, 0.08f), mk(w.v_proj_fc2_b, {od}, 0.05f);
+        moon::model::VisionModel vm(cfg, w);
+        Tensor<uint8_t> img({8, 8, 3});
+        for (auto &px : img.data) px = (uint8_t)((rng_state = rng_state * 6364136223846793005ull + 1442695040888963407ull) >> 56);
+        auto feats = vm.encode_image(img);
+        auto patches = moon::vision::imagePatches(img, 2);
+        Tensor<f16> want({T, od});
+        bool ok = moon_vision_encode_image(vm.session(), patches.data.data(), want.data.data()) == MOON_OK &&
+                  feats.shape == std::vector<size_t>{T, od} && std::memcmp(feats.data.data(), want.data.data(), want.data.size() * sizeof(f16)) == 0;
+        std::vector<float> ff(feats.data.size());
+        orc_cast_f16_to_f32(feats.data.data(), ff.data(), ff.size());
+        double norm = 0;
+        for (float x : ff) ok = ok && std::isfinite(x), norm += (double)x * x;
+        expect(ok && norm > 0, "model.VisionModel.encode_image", norm);
+        auto enc = vm.vision_encoder(patches);
+        expect(enc.shape == std::vector<size_t>{2, T, d}, "model.VisionModel.vision_encoder shape");
+        try {
+            Tensor<f16> one_crop({1, T, pd});
+            vm.vision_encoder(one_crop);
+            expect(false, "one crop must throw");
+        } catch (const moon::InvalidTensorDimension &) { expect(true, "UnexpectedBatchCount"); }
     }
     moon::attention::cleanupThreadPool();
     std::printf("%d failures\n", failures);
