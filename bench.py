@@ -226,8 +226,9 @@ def bench_host_stepped(moon, ctx, model, ids):
     """The reference keeps its generation loop on the host (moondream.zig:323-368).  Two forms of that loop over the
     device-resident session, HOST_STEPS tokens each from the same prefill, wall clock:
       session_calls: next_token() (LM head + arg-max on the device, 4 bytes back) and forward([token]) per token;
-      reference_signatures: what the Zig TextModel drop-in does behind text_decoder / lm_head / text_encoder: a row of
-        embeddings up, the hidden row and the row of logits (100 KB) down, arg-max on the host, the next row looked up."""
+      reference_signatures: the unchanged loop of moondream.zig:323-368 over the drop-ins: text_decoder (a row of embeddings
+        up, the hidden row down), lm_head (100 KB of logits down), the cast to f32, sampling.sample (its drop-in sends the
+        f32 row up again and brings the index back), text_encoder (the next row looked up on the device and brought down)."""
     out = {}
     model.reset()
     model.forward(ids)
@@ -254,12 +255,13 @@ def bench_host_stepped(moon, ctx, model, ids):
         t0 = time.perf_counter()
         for _ in range(n):
             model.text_decoder(x)
-            one[0] = int(np.argmax(model.lm_head()))
+            logits_f32 = model.lm_head().astype(np.float32)  # logits.castWithSimd(f32), moondream.zig:335
+            one[0] = moon.sampling.argmax_f32(logits_f32, ctx=ctx)  # sampling.sample with the greedy method, through its drop-in
             x = model.text_encoder(one)
         dt = time.perf_counter() - t0
-    out["reference_signatures"] = dict(calls_per_token=4, steps=HOST_STEPS, tokens_per_s=HOST_STEPS / dt, ms_per_token=dt / HOST_STEPS * 1e3,
+    out["reference_signatures"] = dict(calls_per_token=5, steps=HOST_STEPS, tokens_per_s=HOST_STEPS / dt, ms_per_token=dt / HOST_STEPS * 1e3,
                                        kv_len_start=model.position - HOST_STEPS,
-                                       bytes_per_token=dict(up=2 * D + 4, down=2 * D + 2 * V + 2 * D))
+                                       bytes_per_token=dict(up=2 * D + 4 * V + 4, down=2 * D + 2 * V + 2 * D + 8))
     return out
 
 
