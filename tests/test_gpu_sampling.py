@@ -377,3 +377,21 @@ def test_quick_walk_never_differs_from_the_exact_walk_next_to_a_boundary(moon, O
     us = us[(us >= 0) & (us < 1)]
     assert us.size >= 40, (m, bounds.size)
     _check(moon, O, ctx, logits, method, us, closed_form=False, **kw)
+
+
+@pytest.mark.parametrize("spread,step", [(3.0, None), (3.0, 0.25), (0.02, None)])
+def test_top_k_in_the_lm_head_kernel_full_vocabulary(moon, O, ctx, spread, step):
+    """The same decision at the real vocabulary (51200 logits over 1024 workgroups, 12 or 13 per wavefront): rows with the
+    logits fixed, 100 draws each, the oracle's index on every draw.  A row quantised to steps of 0.25 has dozens of equal
+    logits at the top (ties inside the three and across their edge: the full evaluation has to take over), a row of spread
+    0.02 has its largest logits within a few f16 steps of each other."""
+    logits = _logits(61, VOCAB, spread=spread, step=step)
+    kw = dict(temperature=0.5, top_k=3)
+    cfg = moon.sampling.sampling_config("top_k", **kw)
+    dev = _fixed_logits_model(moon, O, ctx, logits)
+    us = _boundary_us(O, logits, kw, 100, 62)
+    dev.forward(np.array([5, 6], dtype=np.uint32))
+    got = dev.sample(cfg, us).tolist()
+    want = [O.sample(logits, "top_k", float(u), **kw) for u in us]
+    assert got == want
+    dev.close()
