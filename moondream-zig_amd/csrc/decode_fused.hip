@@ -99,6 +99,27 @@ struct RowGroups {
             if (c + 1 < CH && (c + 1) % chunk == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
     }
+    // pieces [c0, c1) of the one row `first` (and, with c0 == 0, the row's bias), a wait after every `chunk` of them but
+    // the last
+    __device__ __forceinline__ void load_pieces(int first, int lane, int c0, int c1, int chunk) {
+        static_assert(RG == 1, "one row");
+        if (c0 == 0 && lane < RG && first + lane < total) {
+            int m, row;
+            locate(first + lane, m, row);
+            if (bias[m]) bias_lane = bias[m][row];
+        }
+        int m, row;
+        locate(min(first, total - 1), m, row);
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(W[m] + size_t(row) * K);
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            if (c < c0 || c >= c1) continue;
+            const int g = c * 64 + lane;
+            w[0][c] = u32x4{0, 0, 0, 0};
+            if (g < granules && first < total) w[0][c] = __builtin_nontemporal_load(src + g);
+            if (c + 1 < c1 && (c + 1 - c0) % chunk == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+    }
     // done(matrix, row, dot, bias) is called by all lanes
     template <class Done>
     __device__ __forceinline__ void consume(int first, const u32x4 (&xv)[CH], Done done) {
@@ -608,6 +629,11 @@ struct LayerArgs {
     int qkv_wgs;             // workgroups that take qkv rows (the first ones)
     int fc1_rows_out;        // fc1 rows the output workgroups take; the fc1-only workgroups take the rest
 };
+// 1 KiB pieces of an output wavefront's fc2 row that wait in LDS instead of registers (the 80 registers of both rows together
+// do not fit beside the rest, and what the compiler then moves to scratch memory comes back through the memory queue in the
+// last microsecond of the launch)
+constexpr int LAYER_PARK = 4;
+constexpr size_t LAYER_PARK_BYTES = size_t(4) * LAYER_PARK * 64 * 16; // four wavefronts
 constexpr int LAYER_LINE = 32;                       // uint32 per 128-byte line
 constexpr int LAYER_SYNC_HEADS_DONE = 0;             // line 0: heads merged
 constexpr int LAYER_SYNC_FC1_ROOT = 1;               // line 1: fc1 leaves complete
@@ -666,7 +692,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     __shared__ int s_flag;
     constexpr int RG = 4;
     const LnGemvArgs &p = a.g;
-    half_t *s_ln = smem, *s_fc1 = smem + p.d;
+    half_t *s_ln = smem, *s_fc1 = smem + p.d, *s_park = smem + p.d + a.ffn; // (s_park: LAYER_PARK_BYTES)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n_waves = gridDim.x * 4, gw = blockIdx.x * 4 + wave;
     const int n_attn = a.H * DEC_SPLITS, n_out = (p.d + 3) / 4;
@@ -782,19 +808,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     if (!out_wg) return;
 
     // output row of this wavefront; its two weight rows are requested now and arrive during the waits
-    const int n = (b - n_attn) * 4 + wave;
+    const int n = (b - n_attn) * 4 + __builtin_amdgcn_readfirstlane(wave); // (the same in every lane: row addresses stay scalar)
     const bool have_row = n < p.d;
     RowGroups<CH_D, 1> out_row;
     RowGroups<CH_F, 1> fc2_row;
     out_row.init(a.Wo, have_row ? n : 0, have_row ? n + 1 : 0, nullptr, 0, 0, p.d, a.bo);
     fc2_row.init(a.W2, have_row ? n : 0, have_row ? n + 1 : 0, nullptr, 0, 0, a.ffn, a.b2);
     const half_t *hsrc = p.token ? a.hidden_src + size_t(p.token[0]) * p.d : a.hidden_src;
-    half_t hid = (half_t)0.0f;
+    int hid_bits = 0, bias_o_bits = 0, bias_f_bits = 0;
     if (have_row) {
-        hid = hsrc[n];
+        const half_t hid = hsrc[n];
         out_row.load(0, lane);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the out_proj row is in before the fc2 row is asked for
-        fc2_row.load_throttled(0, lane, a.out_chunk);
+        // the first pieces of the fc2 row go to LDS as soon as they are in; the others stay in registers
+        fc2_row.load_pieces(0, lane, 0, LAYER_PARK, CH_F);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // lane 0's old hidden value and the two rows' biases are all here now: as scalars they need no vector register
+        // until the end of the launch
+        hid_bits = __builtin_amdgcn_readfirstlane((int)__builtin_bit_cast(unsigned short, hid));
+        bias_o_bits = __builtin_amdgcn_readfirstlane((int)__builtin_bit_cast(unsigned short, out_row.bias_lane));
+        bias_f_bits = __builtin_amdgcn_readfirstlane((int)__builtin_bit_cast(unsigned short, fc2_row.bias_lane));
+#pragma unroll
+        for (int k = 0; k < LAYER_PARK; k++)
+            *reinterpret_cast<u32x4 *>(s_park + (size_t(wave * LAYER_PARK + k) * 64 + lane) * 8) = fc2_row.w[0][k];
+        fc2_row.load_pieces(0, lane, LAYER_PARK, CH_F, a.out_chunk);
     }
     const unsigned fc1_leaves = n_fc1_wgs < LAYER_FC1_LEAVES ? n_fc1_wgs : LAYER_FC1_LEAVES;
     if (!wait_reached(a.sync + LAYER_SYNC_FC1_ROOT * LAYER_LINE, a.generation * fc1_leaves, a.error, &s_flag)) return;
@@ -807,9 +844,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     for (int i = tid; i < p.d / 4; i += 256) reinterpret_cast<unsigned long long *>(s_attn)[i] = ld_u64_coh(a.attn_out + size_t(i) * 4);
     lds_barrier();
     if (!have_row) return;
-    const half_t bias_o = out_row.bias_lane, bias_f = fc2_row.bias_lane; // lane 0 holds the row's bias
+    const half_t bias_o = __builtin_bit_cast(half_t, (unsigned short)bias_o_bits), bias_f = __builtin_bit_cast(half_t, (unsigned short)bias_f_bits);
+    const half_t hid = __builtin_bit_cast(half_t, (unsigned short)hid_bits);
     const float dot_o = dot_row_lds<CH_D>(out_row.w[0], s_attn, p.d, lane);
-    const float dot_f = dot_row_lds<CH_F>(fc2_row.w[0], s_fc1, a.ffn, lane);
+    float dot_f = 0.0f; // dot_row_lds with the parked pieces read back: the same pieces in the same order
+#pragma unroll
+    for (int c = 0; c < CH_F; c++) {
+        const int g = c * 64 + lane;
+        u32x4 xg = u32x4{0, 0, 0, 0};
+        if (g < (a.ffn >> 3)) xg = *reinterpret_cast<const u32x4 *>(s_fc1 + size_t(g) * 8);
+        const u32x4 wc = c < LAYER_PARK ? *reinterpret_cast<const u32x4 *>(s_park + (size_t(wave * LAYER_PARK + c) * 64 + lane) * 8) : fc2_row.w[0][c];
+        dot_f = dot8(wc, xg, dot_f);
+    }
+    dot_f = wave_sum(dot_f);
     if (lane == 0) {
         const half_t ao = apply_epilogue_v<MOON_EPI_BIAS>(dot_o, bias_o);
         const half_t m = apply_epilogue_v<MOON_EPI_BIAS>(dot_f, bias_f);
@@ -981,9 +1028,9 @@ bool decode_layer_supported(moon_ctx *ctx, size_t d, size_t ffn, size_t H, size_
     int per_cu = 0;
     const void *kernels[2] = {reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 1>), reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 2>)};
     for (const void *k : kernels) {
-        if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)((d + ffn) * sizeof(half_t))) != hipSuccess) return false;
+        if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)((d + ffn) * sizeof(half_t) + LAYER_PARK_BYTES)) != hipSuccess) return false;
         int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k, 256, (d + ffn) * sizeof(half_t)) != hipSuccess) return false;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k, 256, (d + ffn) * sizeof(half_t) + LAYER_PARK_BYTES) != hipSuccess) return false;
         per_cu = per_cu == 0 ? n : std::min(per_cu, n);
     }
     return per_cu * cus > waiting; // producers always find a slot
@@ -1052,8 +1099,8 @@ int launch_decode_layer(moon_ctx *ctx, const half_t *x, const uint32_t *token, c
         const char *e = getenv("MOON_LAYER_FC1_GROUP");
         group = e && atoi(e) == 2 ? 2 : 1;
     }
-    if (group == 2) hipLaunchKernelGGL((decode_layer_kernel<4, 16, 2>), dim3(grid), dim3(256), (d + ffn) * sizeof(half_t), ctx->stream, a);
-    else hipLaunchKernelGGL((decode_layer_kernel<4, 16, 1>), dim3(grid), dim3(256), (d + ffn) * sizeof(half_t), ctx->stream, a);
+    if (group == 2) hipLaunchKernelGGL((decode_layer_kernel<4, 16, 2>), dim3(grid), dim3(256), (d + ffn) * sizeof(half_t) + LAYER_PARK_BYTES, ctx->stream, a);
+    else hipLaunchKernelGGL((decode_layer_kernel<4, 16, 1>), dim3(grid), dim3(256), (d + ffn) * sizeof(half_t) + LAYER_PARK_BYTES, ctx->stream, a);
     MOON_HIP(ctx, hipGetLastError());
     return MOON_OK;
 }
