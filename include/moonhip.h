@@ -425,7 +425,6 @@ int moon_bin_vision_io_weights(const moon_bin *bin, const moon_vision_config *cf
  * diagnostic aids, read once per process unless noted (the first call that looks at them fixes the value for every context):
  *   MOON_DECODE_TRACE=1            text sessions record per-workgroup time stamps of the last layer launch of a greedy call
  *                                  and print a per-role timeline to stderr (allocated at session creation)
- *   MOON_LAYER_OUT_CHUNK=1|2|4|8|16  decode mode 0: 1 KiB pieces of an fc2 row an output wavefront requests before it waits (default 4)
  *   MOON_LAYER_QKV_WGS=n           decode mode 0: workgroups that take qkv rows (default: the attention and output workgroups)
  *   MOON_LAYER_FC1_OUT_ROWS=n      decode mode 0: fc1 rows per output wavefront (default: half an fc1-only wavefront's share)
  *   MOON_LAYER_FC1_GROUP=1|2       decode mode 0: fc1 rows a wavefront requests together (default 1)

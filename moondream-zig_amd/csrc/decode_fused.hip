@@ -79,29 +79,10 @@ struct RowGroups {
             }
         }
     }
-    // load(first) for one-row groups, at most `chunk` pieces in flight: every chunk but the last is waited for before the
-    // next is requested (the shorter the queue in front of a dependent access of this compute unit, the sooner it is served)
-    __device__ __forceinline__ void load_throttled(int first, int lane, int chunk) {
-        static_assert(RG == 1, "one row");
-        if (lane < RG && first + lane < total) {
-            int m, row;
-            locate(first + lane, m, row);
-            if (bias[m]) bias_lane = bias[m][row];
-        }
-        int m, row;
-        locate(min(first, total - 1), m, row);
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(W[m] + size_t(row) * K);
-#pragma unroll
-        for (int c = 0; c < CH; c++) {
-            const int g = c * 64 + lane;
-            w[0][c] = u32x4{0, 0, 0, 0};
-            if (g < granules && first < total) w[0][c] = __builtin_nontemporal_load(src + g);
-            if (c + 1 < CH && (c + 1) % chunk == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        }
-    }
-    // pieces [c0, c1) of the one row `first` (and, with c0 == 0, the row's bias), a wait after every `chunk` of them but
+    // pieces [c0, c1) of the one row `first` (and, with c0 == 0, the row's bias), a wait after every CHUNK of them but
     // the last
-    __device__ __forceinline__ void load_pieces(int first, int lane, int c0, int c1, int chunk) {
+    template <int CHUNK, int SLEEP = 0>
+    __device__ __forceinline__ void load_pieces(int first, int lane, int c0, int c1) {
         static_assert(RG == 1, "one row");
         if (c0 == 0 && lane < RG && first + lane < total) {
             int m, row;
@@ -117,7 +98,11 @@ struct RowGroups {
             const int g = c * 64 + lane;
             w[0][c] = u32x4{0, 0, 0, 0};
             if (g < granules && first < total) w[0][c] = __builtin_nontemporal_load(src + g);
-            if (c + 1 < c1 && (c + 1 - c0) % chunk == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            // A pause between two requests: the pieces wait for the fc1 vector anyway, and the less this wavefront has queued
+            // the sooner the unit's dependent accesses are served (0.622 ms per token with 6 x 64 cycles, 0.632 / 0.628 / 0.640
+            // with 4 / 8 / 10, 0.640-0.650 with none; before, the integer division of a run-time CHUNK happened to fill the gap).
+            if (SLEEP > 0) __builtin_amdgcn_s_sleep(SLEEP);
+            if (c + 1 < c1 && (c + 1 - c0) % CHUNK == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
     }
     // done(matrix, row, dot, bias) is called by all lanes
@@ -625,7 +610,6 @@ struct LayerArgs {
     int H, rot_dim, max_seq, pos, ffn;
     const uint32_t *pos_dev;
     long long *trace;        // optional [grid][8] wall-clock stamps of thread 0 (tuning aid), or null
-    int out_chunk;           // pieces of an output wavefront's fc2 row requested at a time (4, 8 or 16)
     int qkv_wgs;             // workgroups that take qkv rows (the first ones)
     int fc1_rows_out;        // fc1 rows the output workgroups take; the fc1-only workgroups take the rest
 };
@@ -633,6 +617,10 @@ struct LayerArgs {
 // do not fit beside the rest, and what the compiler then moves to scratch memory comes back through the memory queue in the
 // last microsecond of the launch)
 constexpr int LAYER_PARK = 4;
+// 1 KiB pieces of that row requested at a time, each lot waited for before the next is asked for (the shorter the queue in
+// front of a dependent access of this compute unit, the sooner it is served; 2 and 1 measured 3 and 12 % slower, 8 and 16 slower too)
+constexpr int LAYER_OUT_CHUNK = 4;
+constexpr int LAYER_PIECE_SLEEP = 6; // units of 64 cycles between two piece requests (see RowGroups::load_pieces)
 constexpr size_t LAYER_PARK_BYTES = size_t(4) * LAYER_PARK * 64 * 16; // four wavefronts
 constexpr int LAYER_LINE = 32;                       // uint32 per 128-byte line
 constexpr int LAYER_SYNC_HEADS_DONE = 0;             // line 0: heads merged
@@ -821,7 +809,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         out_row.load(0, lane);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the out_proj row is in before the fc2 row is asked for
         // the first pieces of the fc2 row go to LDS as soon as they are in; the others stay in registers
-        fc2_row.load_pieces(0, lane, 0, LAYER_PARK, CH_F);
+        fc2_row.template load_pieces<CH_F, LAYER_PIECE_SLEEP>(0, lane, 0, LAYER_PARK);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         // lane 0's old hidden value and the two rows' biases are all here now: as scalars they need no vector register
         // until the end of the launch
@@ -831,7 +819,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
         for (int k = 0; k < LAYER_PARK; k++)
             *reinterpret_cast<u32x4 *>(s_park + (size_t(wave * LAYER_PARK + k) * 64 + lane) * 8) = fc2_row.w[0][k];
-        fc2_row.load_pieces(0, lane, LAYER_PARK, CH_F, a.out_chunk);
+        fc2_row.template load_pieces<LAYER_OUT_CHUNK, LAYER_PIECE_SLEEP>(0, lane, LAYER_PARK, CH_F);
     }
     const unsigned fc1_leaves = n_fc1_wgs < LAYER_FC1_LEAVES ? n_fc1_wgs : LAYER_FC1_LEAVES;
     if (!wait_reached(a.sync + LAYER_SYNC_FC1_ROOT * LAYER_LINE, a.generation * fc1_leaves, a.error, &s_flag)) return;
@@ -1049,13 +1037,6 @@ int launch_decode_layer(moon_ctx *ctx, const half_t *x, const uint32_t *token, c
     LayerArgs a;
     a.trace = trace;
     {
-        static int chunk = 0;
-        if (!chunk) {
-            const char *e = getenv("MOON_LAYER_OUT_CHUNK");
-            const int v = e ? atoi(e) : 4;
-            chunk = v == 1 || v == 2 || v == 4 || v == 8 ? v : 16;
-        }
-        a.out_chunk = chunk;
         const long long n_attn = (long long)(H * DEC_SPLITS), n_out = (long long)((d + 3) / 4), grid_wgs = (long long)LN_GEMV_GROUPS_PER_CU * (ctx->cu_count > 0 ? ctx->cu_count : 256);
         const long long w_out = n_out * 4, w_fc1 = (grid_wgs - n_attn - n_out) * 4;
         static long long qkv_wgs = -1, r_o = -1;
