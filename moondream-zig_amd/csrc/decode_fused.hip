@@ -839,8 +839,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
     for (int c = 0; c < CH_F; c++) {
         const int g = c * 64 + lane;
-        u32x4 xg = u32x4{0, 0, 0, 0};
-        if (g < (a.ffn >> 3)) xg = *reinterpret_cast<const u32x4 *>(s_fc1 + size_t(g) * 8);
+        // (ffn is a multiple of 512 here, decode_layer_supported: every lane has its piece.  A guarded read would put each
+        // piece behind a branch of its own, and the compiler then keeps all sixteen in registers that are not there.)
+        const u32x4 xg = *reinterpret_cast<const u32x4 *>(s_fc1 + size_t(g) * 8);
         const u32x4 wc = c < LAYER_PARK ? *reinterpret_cast<const u32x4 *>(s_park + (size_t(wave * LAYER_PARK + c) * 64 + lane) * 8) : fc2_row.w[0][c];
         dot_f = dot8(wc, xg, dot_f);
     }
@@ -1008,7 +1009,7 @@ bool decode_fused_supported(size_t d, size_t ffn) {
 
 // Can a whole layer run as one launch of decode_layer_kernel on this device?
 bool decode_layer_supported(moon_ctx *ctx, size_t d, size_t ffn, size_t H, size_t D) {
-    if (D != 64 || pieces(d) != 4 || pieces(ffn) != 16 || H * D != d) return false;
+    if (D != 64 || pieces(d) != 4 || pieces(ffn) != 16 || H * D != d || d % 512 || ffn % 512) return false; // (whole 1 KiB pieces)
     const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
     const int grid = LN_GEMV_GROUPS_PER_CU * cus;
     const int waiting = (int)(H * DEC_SPLITS + (d + 3) / 4); // attention and output workgroups
