@@ -613,15 +613,10 @@ struct LayerArgs {
     int qkv_wgs;             // workgroups that take qkv rows (the first ones)
     int fc1_rows_out;        // fc1 rows the output workgroups take; the fc1-only workgroups take the rest
 };
-// 1 KiB pieces of an output wavefront's fc2 row that wait in LDS instead of registers (the 80 registers of both rows together
-// do not fit beside the rest, and what the compiler then moves to scratch memory comes back through the memory queue in the
-// last microsecond of the launch)
-constexpr int LAYER_PARK = 4;
-// 1 KiB pieces of that row requested at a time, each lot waited for before the next is asked for (the shorter the queue in
+// 1 KiB pieces of an output wavefront's fc2 row requested at a time, each lot waited for before the next is asked for (the shorter the queue in
 // front of a dependent access of this compute unit, the sooner it is served; 2 and 1 measured 3 and 12 % slower, 8 and 16 slower too)
 constexpr int LAYER_OUT_CHUNK = 4;
 constexpr int LAYER_PIECE_SLEEP = 6; // units of 64 cycles between two piece requests (see RowGroups::load_pieces)
-constexpr size_t LAYER_PARK_BYTES = size_t(4) * LAYER_PARK * 64 * 16; // four wavefronts
 constexpr int LAYER_LINE = 32;                       // uint32 per 128-byte line
 constexpr int LAYER_SYNC_HEADS_DONE = 0;             // line 0: heads merged
 constexpr int LAYER_SYNC_FC1_ROOT = 1;               // line 1: fc1 leaves complete
@@ -680,7 +675,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     __shared__ int s_flag;
     constexpr int RG = 4;
     const LnGemvArgs &p = a.g;
-    half_t *s_ln = smem, *s_fc1 = smem + p.d, *s_park = smem + p.d + a.ffn; // (s_park: LAYER_PARK_BYTES)
+    half_t *s_ln = smem, *s_fc1 = smem + p.d;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n_waves = gridDim.x * 4, gw = blockIdx.x * 4 + wave;
     const int n_attn = a.H * DEC_SPLITS, n_out = (p.d + 3) / 4;
@@ -808,18 +803,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         const half_t hid = hsrc[n];
         out_row.load(0, lane);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the out_proj row is in before the fc2 row is asked for
-        // the first pieces of the fc2 row go to LDS as soon as they are in; the others stay in registers
-        fc2_row.template load_pieces<CH_F, LAYER_PIECE_SLEEP>(0, lane, 0, LAYER_PARK);
+        fc2_row.template load_pieces<CH_F, 0>(0, lane, 0, 0); // (no piece yet: the row's bias alone)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         // lane 0's old hidden value and the two rows' biases are all here now: as scalars they need no vector register
         // until the end of the launch
         hid_bits = __builtin_amdgcn_readfirstlane((int)__builtin_bit_cast(unsigned short, hid));
         bias_o_bits = __builtin_amdgcn_readfirstlane((int)__builtin_bit_cast(unsigned short, out_row.bias_lane));
         bias_f_bits = __builtin_amdgcn_readfirstlane((int)__builtin_bit_cast(unsigned short, fc2_row.bias_lane));
-#pragma unroll
-        for (int k = 0; k < LAYER_PARK; k++)
-            *reinterpret_cast<u32x4 *>(s_park + (size_t(wave * LAYER_PARK + k) * 64 + lane) * 8) = fc2_row.w[0][k];
-        fc2_row.template load_pieces<LAYER_OUT_CHUNK, LAYER_PIECE_SLEEP>(0, lane, LAYER_PARK, CH_F);
+        fc2_row.template load_pieces<LAYER_OUT_CHUNK, LAYER_PIECE_SLEEP>(0, lane, 0, CH_F);
     }
     const unsigned fc1_leaves = n_fc1_wgs < LAYER_FC1_LEAVES ? n_fc1_wgs : LAYER_FC1_LEAVES;
     if (!wait_reached(a.sync + LAYER_SYNC_FC1_ROOT * LAYER_LINE, a.generation * fc1_leaves, a.error, &s_flag)) return;
@@ -835,15 +826,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const half_t bias_o = __builtin_bit_cast(half_t, (unsigned short)bias_o_bits), bias_f = __builtin_bit_cast(half_t, (unsigned short)bias_f_bits);
     const half_t hid = __builtin_bit_cast(half_t, (unsigned short)hid_bits);
     const float dot_o = dot_row_lds<CH_D>(out_row.w[0], s_attn, p.d, lane);
-    float dot_f = 0.0f; // dot_row_lds with the parked pieces read back: the same pieces in the same order
+    float dot_f = 0.0f; // dot_row_lds without its guards
 #pragma unroll
     for (int c = 0; c < CH_F; c++) {
         const int g = c * 64 + lane;
         // (ffn is a multiple of 512 here, decode_layer_supported: every lane has its piece.  A guarded read would put each
         // piece behind a branch of its own, and the compiler then keeps all sixteen in registers that are not there.)
         const u32x4 xg = *reinterpret_cast<const u32x4 *>(s_fc1 + size_t(g) * 8);
-        const u32x4 wc = c < LAYER_PARK ? *reinterpret_cast<const u32x4 *>(s_park + (size_t(wave * LAYER_PARK + c) * 64 + lane) * 8) : fc2_row.w[0][c];
-        dot_f = dot8(wc, xg, dot_f);
+        dot_f = dot8(fc2_row.w[0][c], xg, dot_f);
     }
     dot_f = wave_sum(dot_f);
     if (lane == 0) {
@@ -1017,9 +1007,9 @@ bool decode_layer_supported(moon_ctx *ctx, size_t d, size_t ffn, size_t H, size_
     int per_cu = 0;
     const void *kernels[2] = {reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 1>), reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 2>)};
     for (const void *k : kernels) {
-        if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)((d + ffn) * sizeof(half_t) + LAYER_PARK_BYTES)) != hipSuccess) return false;
+        if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)((d + ffn) * sizeof(half_t))) != hipSuccess) return false;
         int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k, 256, (d + ffn) * sizeof(half_t) + LAYER_PARK_BYTES) != hipSuccess) return false;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k, 256, (d + ffn) * sizeof(half_t)) != hipSuccess) return false;
         per_cu = per_cu == 0 ? n : std::min(per_cu, n);
     }
     return per_cu * cus > waiting; // producers always find a slot
@@ -1081,8 +1071,8 @@ int launch_decode_layer(moon_ctx *ctx, const half_t *x, const uint32_t *token, c
         const char *e = getenv("MOON_LAYER_FC1_GROUP");
         group = e && atoi(e) == 2 ? 2 : 1;
     }
-    if (group == 2) hipLaunchKernelGGL((decode_layer_kernel<4, 16, 2>), dim3(grid), dim3(256), (d + ffn) * sizeof(half_t) + LAYER_PARK_BYTES, ctx->stream, a);
-    else hipLaunchKernelGGL((decode_layer_kernel<4, 16, 1>), dim3(grid), dim3(256), (d + ffn) * sizeof(half_t) + LAYER_PARK_BYTES, ctx->stream, a);
+    if (group == 2) hipLaunchKernelGGL((decode_layer_kernel<4, 16, 2>), dim3(grid), dim3(256), (d + ffn) * sizeof(half_t), ctx->stream, a);
+    else hipLaunchKernelGGL((decode_layer_kernel<4, 16, 1>), dim3(grid), dim3(256), (d + ffn) * sizeof(half_t), ctx->stream, a);
     MOON_HIP(ctx, hipGetLastError());
     return MOON_OK;
 }
