@@ -29,20 +29,25 @@ constexpr int DEC_PREFETCH = 4;                 // keys per lane group whose K a
 // Merge the DEC_SPLITS partials of one head in a fixed order; returns output element d of that head.
 template <int D, bool COH = false>
 __device__ __forceinline__ half_t decode_attn_merge(const float *__restrict__ p /* partials of this head */, int d) {
-    float ms_[DEC_SPLITS];
-    float m = -INFINITY;
+    // everything is requested before anything is used: one round trip (device-coherent loads are issued where the source
+    // has them, so loads that followed the maximum would be a second one)
+    float ms_[DEC_SPLITS], ls_[DEC_SPLITS], os_[DEC_SPLITS];
 #pragma unroll
     for (int s = 0; s < DEC_SPLITS; s++) {
         ms_[s] = ld_f<COH>(p + s * (D + 2) + D);
-        m = fmaxf(m, ms_[s]);
+        ls_[s] = ld_f<COH>(p + s * (D + 2) + D + 1);
+        os_[s] = ld_f<COH>(p + s * (D + 2) + d);
     }
+    float m = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < DEC_SPLITS; s++) m = fmaxf(m, ms_[s]);
     float l = 0.0f, o = 0.0f;
 #pragma unroll
     for (int s = 0; s < DEC_SPLITS; s++) {
         const float ms = ms_[s];
         const float w = (ms == -INFINITY) ? 0.0f : __expf(ms - m);
-        l = fmaf(ld_f<COH>(p + s * (D + 2) + D + 1), w, l);
-        o = fmaf(ld_f<COH>(p + s * (D + 2) + d), w, o);
+        l = fmaf(ls_[s], w, l);
+        o = fmaf(os_[s], w, o);
     }
     return (half_t)f32_round(o * (1.0f / l)); // attention.zig:612-615 multiplies by the reciprocal of the sum
 }

@@ -652,6 +652,13 @@ __device__ __forceinline__ bool wait_reached(uint32_t *word, uint32_t target, ui
     return *s_flag != 0;
 }
 
+
+// 16 bytes, device-coherent, waited for on the spot (p 16-byte aligned)
+__device__ __forceinline__ u32x4 ld_u128_coh(const void *p) {
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
 // dot of the loaded row (group slot 0) with a vector that lives in LDS, pieces in the same order as RowGroups::consume
 template <int CH>
 __device__ __forceinline__ float dot_row_lds(const u32x4 (&w)[CH], const half_t *x_lds, int K, int lane) {
@@ -820,7 +827,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     if (!wait_reached(a.sync + LAYER_SYNC_HEADS_DONE * LAYER_LINE, a.generation * (uint32_t)a.H, a.error, &s_flag)) return;
     stamp(4); // all heads merged
     half_t *s_attn = s_ln; // the LayerNorm output is no longer needed
-    for (int i = tid; i < p.d / 4; i += 256) reinterpret_cast<unsigned long long *>(s_attn)[i] = ld_u64_coh(a.attn_out + size_t(i) * 4);
+    // (one 16-byte load per thread: this copy is the last hop of the launch.  The fc1 vector above is better off in 8-byte
+    // loads, whose waits space out the requests: 0.628 ms per token with 16-byte ones there, 0.598 as it is, 0.602 with both in
+    // 8-byte loads; an agent-scope acquire followed by plain loads, so that the die's L2 serves 63 of its 64 workgroups: 0.91 ms)
+    for (int i = tid; i < p.d / 8; i += 256) reinterpret_cast<u32x4 *>(s_attn)[i] = ld_u128_coh(a.attn_out + size_t(i) * 8);
     lds_barrier();
     if (!have_row) return;
     const half_t bias_o = __builtin_bit_cast(half_t, (unsigned short)bias_o_bits), bias_f = __builtin_bit_cast(half_t, (unsigned short)bias_f_bits);
