@@ -585,7 +585,7 @@ __global__ __launch_bounds__(256) void decode_front_kernel(FrontArgs a) {
 //   [A, A + O)         O = d / 4 output workgroups (one hidden element per wavefront): a few fc1 rows, then the
 //                      wavefront requests its out_proj row and its fc2 row (20 KiB, in flight during the waits), waits
 //                      for "all fc1 rows written" and "all heads done", and writes hidden += out_proj(attn) + fc2(fc1)
-//   [A + O, grid)      the remaining fc1 rows (twice as many per wavefront as the output workgroups take)
+//   [A + O, grid)      the remaining fc1 rows (several times as many per wavefront as the output workgroups take)
 // The weight stream of a later phase is always requested before the wait for the earlier phase's vector, so HBM stays
 // busy across the three dependent exchanges that otherwise cost a kernel launch each.  Arithmetic, rounding points and
 // summation orders are those of the separate kernels: the results are bit-identical.
@@ -760,7 +760,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         return;
     }
 
-    // fc1 rows: output wavefronts take one share each, the fc1-only wavefronts two
+    // fc1 rows: the output wavefronts take fc1_rows_out of them between themselves, the fc1-only wavefronts the rest
     {
         int b0, b1;
         const int w_out = n_out * 4, w_fc1 = (gridDim.x - n_attn - n_out) * 4;
@@ -1045,12 +1045,17 @@ int launch_decode_layer(moon_ctx *ctx, const half_t *x, const uint32_t *token, c
             const char *e = getenv("MOON_LAYER_QKV_WGS");
             qkv_wgs = e ? atoll(e) : 0;
             const char *f = getenv("MOON_LAYER_FC1_OUT_ROWS");
-            r_o = f ? atoll(f) : 0;
+            r_o = f ? atoll(f) + 1 : 0; // (kept as rows + 1 so that 0 rows can be asked for)
         }
         // by default the fc1-only workgroups, the last to be served on every compute unit, take no qkv rows
         const long long qkv_default = 3 * (long long)d <= 64 * (n_attn + n_out) ? n_attn + n_out : grid_wgs;
+        // an fc1-only wavefront takes about three times the fc1 rows of an output wavefront, which has its 20 KiB of out_proj
+        // and fc2 rows to request as well; whole rows per output wavefront, at least one (moondream: 1 and 6 rows; 2 and 4
+        // measured 0.598 against 0.592 ms per token, none and 8 0.673)
+        const long long per_out_wave = w_fc1 > 0 ? std::max<long long>(1, (long long)ffn / (w_out + 3 * w_fc1)) : (long long)ffn;
+        const long long default_rows_out = std::min<long long>((long long)ffn, w_out * per_out_wave);
         a.qkv_wgs = (int)(qkv_wgs > 0 && qkv_wgs <= grid_wgs && 3 * (long long)d <= 64 * qkv_wgs ? qkv_wgs : qkv_default);
-        a.fc1_rows_out = (int)(r_o > 0 && w_fc1 > 0 ? std::min<long long>((long long)ffn, w_out * r_o) : (long long)ffn * w_out / (w_out + 2 * w_fc1));
+        a.fc1_rows_out = (int)(r_o > 0 && w_fc1 > 0 ? std::min<long long>((long long)ffn, w_out * (r_o - 1)) : default_rows_out);
     }
     a.g = LnGemvArgs{x, token, gamma, beta, Wqkv, bqkv, qkv, W1, b1, fc1, (int)d, (int)(3 * d), (int)ffn, eps};
     a.Wo = Wo;
