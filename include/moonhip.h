@@ -426,13 +426,17 @@ int moon_bin_vision_io_weights(const moon_bin *bin, const moon_vision_config *cf
  *   MOON_DECODE_TRACE=1            text sessions record per-workgroup time stamps of the last layer launch of a greedy call
  *                                  and print a per-role timeline to stderr (allocated at session creation)
  *   MOON_LAYER_QKV_WGS=n           decode mode 0: workgroups that take qkv rows (default: the attention and output workgroups)
- *   MOON_LAYER_FC1_OUT_ROWS=n      decode mode 0: fc1 rows per output wavefront (default: half an fc1-only wavefront's share)
+ *   MOON_LAYER_FC1_OUT_ROWS=n      decode mode 0: fc1 rows per output wavefront (default: about a third of an fc1-only wavefront's
+ *                                  share, at least one; 0 is allowed)
  *   MOON_LAYER_FC1_GROUP=1|2       decode mode 0: fc1 rows a wavefront requests together (default 1)
  *   MOON_GEMM_KERNEL=regs|dma|dma256|w114|w212|w221  forces one of the MFMA product kernels where the shape allows it (default: by shape)
  *   MOON_GEMM_EPILOGUE=direct      the product kernels store their tile without the pass through LDS (default: through LDS)
  *   MOON_SAMPLE_SEPARATE=1         sampled loops with top_k <= 3: the LM-head launch leaves every token to sample_kernel instead of
  *                                  deciding it where it provably can (read at every call, so a test can compare the two in one process)
- * Every setting gives the same results, bit for bit; only the time changes. */
+ *   MOON_GEMM_NO_PAIR=1            text prefill: a block's out_proj and fc2 run as launches of their own instead of one joint launch
+ *                                  (read at every call); the two forms split K differently, so their f32 sums, and with them a few
+ *                                  f16 roundings, differ
+ * Every other setting gives the same results, bit for bit; only the time changes. */
 
 #ifdef __cplusplus
 }

@@ -108,13 +108,13 @@ __device__ __forceinline__ void gemm_store_tile_lds(const GemmArgs &p, const flo
 
 // A wavefront's 64x64 f32 partial tile of a split K, written in full lines the same way: half of the tile (32 rows m) at a
 // time through 32 * 68 floats of LDS, four consecutive n per lane on the way out.  Needs N % 4 == 0.
-template <int EPI>
-__device__ __forceinline__ void gemm_store_partial_lds(const GemmArgs &p, const float16_t (&acc)[2][2], int m0, int n0, int wm, int wn, int lane,
+template <int EPI, int MB = 2> // MB: 32-row blocks of m in the sub-tile, as in gemm_store_tile_lds
+__device__ __forceinline__ void gemm_store_partial_lds(const GemmArgs &p, const float16_t (&acc)[2][MB], int m0, int n0, int wm, int wn, int lane,
                                                        int split, float *scratch) {
     const int frag_row = lane & 31, frag_g = lane >> 5;
     const int nl = (lane & 15) * 4, n = n0 + wn * 64 + nl;
 #pragma unroll
-    for (int mi = 0; mi < 2; mi++) {
+    for (int mi = 0; mi < MB; mi++) {
 #pragma unroll
         for (int ni = 0; ni < 2; ni++)
 #pragma unroll
@@ -510,22 +510,25 @@ template <int MI> struct Dma2 {
     static constexpr int A_LOADS = 2 * MI; // copies of activation rows per loader wavefront and k-tile (8 rows each)
 };
 
-template <int EPI, int MI>
-__device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p) {
+// PARTIAL: the workgroup multiplies k-tiles [kt0, kt0 + n_ktiles) of tile `wg` only and leaves the f32 sums in slab `split` of
+// p.partial (no epilogue); otherwise the whole of K, and wg is taken from the workgroup index.
+template <int EPI, int MI, bool PARTIAL = false>
+__device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p, int wg_arg = 0, int kt0 = 0, int n_ktiles_arg = 0, int split = 0) {
     static_assert(MI == 3 || MI == 4, "192- or 256-row tiles");
+    static_assert(!PARTIAL || EPI == MOON_EPI_NONE, "partial sums take no epilogue");
     constexpr int BM2 = Dma2<MI>::BM2, STAGE2_HALFS = Dma2<MI>::STAGE2_HALFS, A_LOADS = Dma2<MI>::A_LOADS;
-    constexpr bool SHARED_EPILOGUE = EPI == MOON_EPI_BIAS_GELU; // all eight wavefronts finish the tile
+    constexpr bool SHARED_EPILOGUE = EPI == MOON_EPI_BIAS_GELU && !PARTIAL; // all eight wavefronts finish the tile
     static_assert(size_t(BM2) * TILE_PITCH <= size_t(DMA2_STAGES) * STAGE2_HALFS, "the parked tile fits the staging area");
     extern __shared__ __attribute__((aligned(16))) half_t lds2[]; // [stage][act: 256 rows | weight: 128 rows][64 halfs]
 
     const int total = p.tiles_m * p.tiles_n;
     const int per_xcd = (total + 7) / 8;
     // (workgroup id -> tile as in the 128 x 128 kernel: the ids an XCD receives cover a contiguous run of tiles)
-    const int wg = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    const int wg = PARTIAL ? wg_arg : (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (wg >= total) return;
     const int tn = wg / p.tiles_m, tm = wg % p.tiles_m;
     const int m0 = tm * BM2, n0 = tn * BN;
-    const int n_ktiles = p.K / BK;
+    const int n_ktiles = PARTIAL ? n_ktiles_arg : p.K / BK;
 
     const int t = threadIdx.x, lane = t & 63;
     const int role_wave = (t >> 6) & 3;
@@ -549,7 +552,7 @@ __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p) {
         }
         auto issue = [&](int kt) {
             half_t *stage = lds2 + size_t(kt % DMA2_STAGES) * STAGE2_HALFS;
-            const int k_off = kt * BK * 2;
+            const int k_off = (kt0 + kt) * BK * 2;
 #pragma unroll
             for (int j = 0; j < A_LOADS; j++)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (__attribute__((address_space(3))) void *)(stage + (16 * MI * role_wave + 8 * j) * BK),
@@ -686,6 +689,33 @@ __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p) {
         gemm_tile_out<EPI, BM2>(p, m0, n0, t, lds2);
         return;
     }
+    if constexpr (PARTIAL) {
+        // the stage after the last k-tile's is free (every copy into it has landed and been read): 32 x 68 floats per wavefront
+        float *fscratch = reinterpret_cast<float *>(lds2 + size_t(n_ktiles % DMA2_STAGES) * STAGE2_HALFS) + size_t(role_wave) * 32 * EPI_PITCH;
+        static_assert(size_t(4) * 32 * EPI_PITCH * sizeof(float) <= size_t(STAGE2_HALFS) * sizeof(half_t), "the four wavefronts' slots fit a stage");
+        {
+            float16_t part[2][2];
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                for (int mi = 0; mi < 2; mi++) part[ni][mi] = acc[ni][mi];
+            gemm_store_partial_lds<EPI>(p, part, m0 + wm * 32 * MI - wm * 64, n0, wm, wn, lane, split, fscratch);
+        }
+        if constexpr (MI == 4) {
+            float16_t part[2][2];
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                for (int mi = 0; mi < 2; mi++) part[ni][mi] = acc[ni][MI - 2 + mi];
+            gemm_store_partial_lds<EPI>(p, part, m0 + wm * 32 * MI + 64 - wm * 64, n0, wm, wn, lane, split, fscratch);
+        } else {
+            float16_t part[2][1];
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++) part[ni][0] = acc[ni][MI - 1];
+            gemm_store_partial_lds<EPI, 1>(p, part, m0 + wm * 32 * MI + 64 - wm * 64, n0, wm, wn, lane, split, fscratch);
+        }
+        return;
+    }
     // the stage after the last k-tile's is free (every copy into it has landed and been read): 64 x 68 halfs per wavefront
     half_t *scratch = lds2 + size_t(n_ktiles % DMA2_STAGES) * STAGE2_HALFS + size_t(role_wave) * 64 * EPI_PITCH;
     { // the first 64 rows of the sub-tile
@@ -719,6 +749,28 @@ __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma256_kernel(GemmArgs p)
 template <int EPI>
 __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma192_kernel(GemmArgs p) {
     gemm_nt_dma2_body<EPI, 3>(p);
+}
+
+// TWO products with the same [M, N] result shape in one launch, each with its own split of K, f32 partial sums only (the
+// decoder block's out_proj and fc2, whose results are added: text_model.zig:163-171).  Alone, each of them leaves a
+// quarter of the compute units idle at 768 rows (192 workgroups); together their 192 x 128 tiles times the splits fill all of
+// them.  Workgroups [0, units0) take problem 0 (tile = unit % tiles, split = unit / tiles), the others problem 1.
+struct GemmPairArgs {
+    GemmArgs p[2];
+    int units0, units_total;
+};
+__global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma192_pair_kernel(GemmPairArgs a) {
+    const int per_xcd = (a.units_total + 7) / 8;
+    const int unit = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (unit >= a.units_total) return;
+    const bool first = unit < a.units0;
+    const GemmArgs &p = first ? a.p[0] : a.p[1];
+    const int u = first ? unit : unit - a.units0;
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int split = u / tiles, tile = u % tiles;
+    const int k_begin = split * p.k_per_split, k_end = min(p.K, k_begin + p.k_per_split);
+    if (k_end <= k_begin) return;
+    gemm_nt_dma2_body<MOON_EPI_NONE, 3, true>(p, tile, k_begin / BK, (k_end - k_begin) / BK, split);
 }
 
 template <int EPI>
@@ -1162,6 +1214,79 @@ int launch_gemm_partials(moon_ctx *ctx, const half_t *A, const half_t *B, size_t
         return MOON_OK;
     }
     return rc;
+}
+
+int launch_gemm_pair_ln(moon_ctx *ctx, const half_t *A_add, const half_t *B_add, const half_t *bias_add, size_t K_add, const half_t *A, const half_t *B,
+                        const half_t *bias, size_t K, const half_t *resid, half_t *C, size_t M, size_t N, const GemmLayerNorm &ln, bool *done) {
+    *done = false;
+    const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    const size_t buf_max = (size_t(1) << 31) - 4096;
+    const auto al16 = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+    if (ctx->gemm_kernel[0] || getenv("MOON_GEMM_NO_PAIR")) return MOON_OK; // (a kernel was named for measurements: the products run one by one)
+    if (M < 192 || M > 0x3fffffff || N % 8 || N > (size_t)LN_FUSE_MAX_N || K % BK || K_add % BK || !K || !K_add) return MOON_OK;
+    if (M * K * 2 >= buf_max || N * K * 2 >= buf_max || M * K_add * 2 >= buf_max || N * K_add * 2 >= buf_max) return MOON_OK;
+    if (!al16(A) || !al16(B) || !al16(A_add) || !al16(B_add) || !al16(bias) || !al16(bias_add) || !al16(resid) || !al16(C) || !al16(ln.gamma) ||
+        !al16(ln.beta) || !al16(ln.out) || !ln.add || !al16(ln.add))
+        return MOON_OK;
+    const int tiles_m = (int)((M + 191) / 192), tiles_n = (int)((N + BN - 1) / BN), tiles = tiles_m * tiles_n;
+    if (tiles * 2 > cus) return MOON_OK;
+    // splits (s_add, s): all workgroups in one round, the longest run of k-tiles as short as it gets
+    const int kt_add = (int)(K_add / BK), kt = (int)(K / BK);
+    int best_a = 0, best_s = 0, best_len = 1 << 30;
+    for (int sa = 1; sa <= 8 && sa <= kt_add; sa++)
+        for (int s = 1; s <= 8 && s <= kt; s++) {
+            if (tiles * (sa + s) > cus) continue;
+            const int len = std::max((kt_add + sa - 1) / sa, (kt + s - 1) / s);
+            if (len < best_len || (len == best_len && sa + s < best_a + best_s)) {
+                best_len = len;
+                best_a = sa;
+                best_s = s;
+            }
+        }
+    if (!best_a) return MOON_OK;
+    GemmPairArgs a;
+    const auto fill = [&](GemmArgs &p, const half_t *Ap, const half_t *Bp, size_t Kp, int splits, GrowBuf &ws) -> int {
+        p.A = Ap;
+        p.Bt = Bp;
+        p.bias = nullptr;
+        p.resid = nullptr;
+        p.C = nullptr;
+        p.M = (int)M;
+        p.N = (int)N;
+        p.K = (int)Kp;
+        p.tiles_m = tiles_m;
+        p.tiles_n = tiles_n;
+        const int ktp = (int)(Kp / BK);
+        p.k_per_split = (ktp + splits - 1) / splits * BK;
+        p.splits = (int)((Kp + p.k_per_split - 1) / p.k_per_split);
+        p.a_bytes = (int)(M * Kp * 2);
+        p.bt_bytes = (int)(N * Kp * 2);
+        p.lds_epilogue = 1;
+        p.super_m = p.super_n = 1;
+        MOON_TRY(moon_grow(ctx, ws, size_t(p.splits) * M * N * sizeof(float)));
+        p.partial = (float *)ws.ptr;
+        return MOON_OK;
+    };
+    MOON_TRY(fill(a.p[0], A_add, B_add, K_add, best_a, ctx->work[3]));
+    MOON_TRY(fill(a.p[1], A, B, K, best_s, ctx->work[0]));
+    a.units0 = tiles * a.p[0].splits;
+    a.units_total = a.units0 + tiles * a.p[1].splits;
+    static std::atomic<bool> attr_set[64];
+    const int dev = ctx->device >= 0 && ctx->device < 64 ? ctx->device : -1;
+    if (dev < 0 || !attr_set[dev].load()) {
+        MOON_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_nt_dma192_pair_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)Dma2<3>::LDS_BYTES));
+        if (dev >= 0) attr_set[dev].store(true);
+    }
+    hipLaunchKernelGGL(gemm_nt_dma192_pair_kernel, dim3(((a.units_total + 7) / 8) * 8), dim3(DMA_THREADS), Dma2<3>::LDS_BYTES, ctx->stream, a);
+    MOON_NOTE_KERNEL(ctx, "gemm_nt_dma192_pair_kernel %d + %d workgroups, k splits %d and %d + splitk_reduce_ln_kernel", a.units0, a.units_total - a.units0,
+                     a.p[0].splits, a.p[1].splits);
+    MOON_HIP(ctx, hipGetLastError());
+    hipLaunchKernelGGL(splitk_reduce_ln_kernel<MOON_EPI_BIAS_RESID>, dim3((unsigned)M), dim3(256), 0, ctx->stream, a.p[1].partial, bias, resid, ln.add,
+                       a.p[0].partial, a.p[0].splits, bias_add, C, ln.gamma, ln.beta, ln.out, (int)M, (int)N, a.p[1].splits, ln.eps);
+    MOON_HIP(ctx, hipGetLastError());
+    *done = true;
+    return MOON_OK;
 }
 
 // dst[cols, rows] = src[rows, cols]^T

@@ -124,6 +124,13 @@ int launch_gemm_partials(moon_ctx *ctx, const half_t *A, const half_t *B, size_t
                          int *splits);
 int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias, half_t *C,
                 size_t M, size_t N, size_t K, int b_layout, int epilogue, const half_t *resid = nullptr, const GemmLayerNorm *ln = nullptr);
+// Two products with the same [M, N] result in ONE launch, then the launch that finishes both, as launch_gemm does with
+// ln->add_partial set: C = f16(resid + f16(add + t)), add = f16(f16(A_add . B_add^T) + bias_add), t = f16(f16(A . B^T) + bias),
+// and the LayerNorm of the finished rows into ln.out (ln.add must name M x N halfs all the same).  Both B operands are [N, K].
+// Only for shapes where that fills the device in one round (M >= 192, N <= 2048, K's multiples of 64, 16-byte aligned
+// operands); *done says whether anything was launched, and if not the caller runs the products one by one.
+int launch_gemm_pair_ln(moon_ctx *ctx, const half_t *A_add, const half_t *B_add, const half_t *bias_add, size_t K_add, const half_t *A, const half_t *B,
+                        const half_t *bias, size_t K, const half_t *resid, half_t *C, size_t M, size_t N, const GemmLayerNorm &ln, bool *done);
 
 int launch_layernorm(moon_ctx *ctx, const half_t *x, const half_t *gamma, const half_t *beta, half_t *y,
                      size_t rows, size_t dim, float eps);

@@ -311,23 +311,29 @@ int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool p
         MOON_TRY(launch_qkv_rope_cache(ctx, m->qkv, m->q_rot, ck, cv, m->freqs, n, z.H, z.D, m->cfg.rot_dim, z.S, pos));
         MOON_TRY(launch_sdpa(ctx, m->q_rot, ck, cv, m->attn, z.H, n, pos + n, z.D, z.S * z.D, (long)pos, nullptr, 0, true));
         const bool finish_in_fc2 = chain_ln && layer + 1 < z.L;
-        // where fc2 finishes the block, out_proj leaves its split-K partials for that launch to reduce as well
-        const float *out_partial = nullptr;
-        int out_splits = 0;
-        if (finish_in_fc2) MOON_TRY(launch_gemm_partials(ctx, m->attn, out_w, n, z.d, z.d, MOON_B_NK, &out_partial, &out_splits));
-        if (!out_splits) MOON_TRY(launch_gemm(ctx, m->attn, out_w, out_b, m->attn_proj, n, z.d, z.d, MOON_B_NK, MOON_EPI_BIAS));
-        MOON_TRY(launch_gemm(ctx, m->ln_in, fc1_w, fc1_b, m->fc1, n, z.ffn, z.d, MOON_B_NK, MOON_EPI_BIAS_GELU));
         if (finish_in_fc2) {
+            // out_proj and fc2 as one launch (each alone leaves a quarter of the device idle at 768 rows), finished together
+            MOON_TRY(launch_gemm(ctx, m->ln_in, fc1_w, fc1_b, m->fc1, n, z.ffn, z.d, MOON_B_NK, MOON_EPI_BIAS_GELU));
             GemmLayerNorm next{m->ln_w + (layer + 1) * z.d, m->ln_b + (layer + 1) * z.d, m->ln_in, m->cfg.ln_eps};
             next.add = m->attn_proj;
             next.add_scratch = m->mlp;
-            if (out_splits) {
+            bool done = false;
+            MOON_TRY(launch_gemm_pair_ln(ctx, m->attn, out_w, out_b, z.d, m->fc1, fc2_w, fc2_b, z.ffn, m->hidden, m->hidden, n, z.d, next, &done));
+            if (done) return MOON_OK;
+            // (otherwise the products one by one; fc1 is in place already)
+            const float *out_partial = nullptr;
+            int out_splits = 0;
+            MOON_TRY(launch_gemm_partials(ctx, m->attn, out_w, n, z.d, z.d, MOON_B_NK, &out_partial, &out_splits));
+            if (!out_splits) MOON_TRY(launch_gemm(ctx, m->attn, out_w, out_b, m->attn_proj, n, z.d, z.d, MOON_B_NK, MOON_EPI_BIAS));
+            else {
                 next.add_partial = out_partial;
                 next.add_splits = out_splits;
                 next.add_bias = out_b;
             }
             return launch_gemm(ctx, m->fc1, fc2_w, fc2_b, m->hidden, n, z.d, z.ffn, MOON_B_NK, 3 /* bias, then += into hidden */, m->hidden, &next);
         }
+        MOON_TRY(launch_gemm(ctx, m->attn, out_w, out_b, m->attn_proj, n, z.d, z.d, MOON_B_NK, MOON_EPI_BIAS));
+        MOON_TRY(launch_gemm(ctx, m->ln_in, fc1_w, fc1_b, m->fc1, n, z.ffn, z.d, MOON_B_NK, MOON_EPI_BIAS_GELU));
         MOON_TRY(launch_gemm(ctx, m->fc1, fc2_w, fc2_b, m->mlp, n, z.d, z.ffn, MOON_B_NK, MOON_EPI_BIAS));
     }
     return launch_residual2(ctx, m->hidden, m->attn_proj, m->mlp, n * z.d);

@@ -237,6 +237,30 @@ def test_decode_modes_agree_full_size(moon, O, ctx):
     dev.close()
 
 
+def test_prefill_with_out_proj_and_fc2_in_one_launch(moon, O, ctx, monkeypatch):
+    """At 192 rows and more the prefill runs a block's out_proj and fc2 as ONE launch (their partial sums are finished
+    together); MOON_GEMM_NO_PAIR keeps them apart.  Same arithmetic but other splits of K.  Three layers of the real width
+    (the first two take the joint launch) on a ragged prompt (333 rows: the last row block of the 192-row tiles is partial):
+    both forms match the oracle, agree with each other, and are not the same bits (which they would be if the joint launch
+    had not been taken)."""
+    cfg = dict(O.TEXT_CFG, n_layers=3, vocab=2048)
+    ref, dev = _text_pair(moon, O, ctx, cfg, seed=4)
+    ids = O.fill_uniform_u32(333, 0, 51, cfg["vocab"])
+    h_ref = ref.text_decoder(ref.text_encoder(ids), ref.new_cache())
+    dev.forward(ids)
+    h_pair = dev.hidden(333).copy()
+    monkeypatch.setenv("MOON_GEMM_NO_PAIR", "1")
+    dev.reset()
+    dev.forward(ids)
+    h_one = dev.hidden(333).copy()
+    monkeypatch.delenv("MOON_GEMM_NO_PAIR")
+    dev.close()
+    assert not np.array_equal(h_pair.view(np.uint16), h_one.view(np.uint16))
+    errs = O.rel_frobenius(h_pair, h_ref), O.rel_frobenius(h_one, h_ref), O.rel_frobenius(h_pair, h_one)
+    print("\njoint launch / separate launches against the oracle, and against each other: %.2e %.2e %.2e" % errs, flush=True)
+    assert max(errs) <= TOL
+
+
 def test_sessions_built_from_a_moondream_bin_file(moon, O, ctx, tmp_path):
     """Weights written in the reference's file layout, mapped by the library's reader and uploaded from the mapping: the
     decoder and the vision encoder give the same bits as when built from in-memory arrays, and match the oracle."""
