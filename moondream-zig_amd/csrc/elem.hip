@@ -110,13 +110,6 @@ __global__ void rope_table_kernel(float *table, int half_pairs, int end, int dim
     table[2 * i + 1] = (float)sin((double)ang);
 }
 
-__device__ __forceinline__ void rotate_pair(float xr, float xi, float c, float s, half_t &o_r, half_t &o_i) {
-#pragma clang fp contract(off)
-    // rope.zig:223-224, separate multiplies and adds
-    o_r = (half_t)(xr * c - xi * s);
-    o_i = (half_t)(xr * s + xi * c);
-}
-
 // rope.applyRotEmb (rope.zig:130-272) on [H,S,D]; one thread per (h,s,d<D) element slot
 __global__ void rope_apply_kernel(const half_t *__restrict__ x, half_t *__restrict__ out, int H, int S, int D,
                                   const float *__restrict__ table, const uint64_t *__restrict__ position_ids,

@@ -49,6 +49,13 @@ __device__ __forceinline__ half_t apply_epilogue(float acc, const half_t *__rest
     return apply_epilogue_v<EPI>(acc, EPI >= MOON_EPI_BIAS ? bias[n] : (half_t)0.0f);
 }
 
+// One rotation of rope.applyRotEmb (rope.zig:223-224): separate multiplies and adds, one rounding to f16 each
+__device__ __forceinline__ void rotate_pair(float xr, float xi, float c, float s, half_t &o_r, half_t &o_i) {
+#pragma clang fp contract(off)
+    o_r = (half_t)(xr * c - xi * s);
+    o_i = (half_t)(xr * s + xi * c);
+}
+
 // Workgroup barrier for data exchanged through LDS only: waits for this wavefront's LDS operations, not for its
 // outstanding global loads (which __syncthreads() would drain), so prefetched weights stay in flight across it.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }

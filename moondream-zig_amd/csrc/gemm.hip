@@ -281,6 +281,58 @@ __device__ __forceinline__ void gemm_tile_out(const GemmArgs &p, int m0, int n0,
     }
 }
 
+// gemm_tile_out for a qkv projection, with what qkv_rope_cache_vec_kernel does to the finished rows folded in (the same
+// values, roundings and rotations: the results are the same bits), so that the projection never goes to memory unrotated.
+// The tile's 128 columns are two whole heads of q, k or v (heads are 64 wide, tiles start at multiples of 128).  A thread
+// finishes eight consecutive columns of a row; where those are rotated it also forms the eight partner values, rot_dim / 2
+// further on or back in the same head, from the parked tile and their bias.
+template <int ROWS>
+__device__ __forceinline__ void gemm_tile_out_rope(const GemmArgs &p, int m0, int n0, int t, const half_t *scratch) {
+    const int nl = (t & 15) * 8, n = n0 + nl, d0 = nl & 63; // d0: first of the eight columns within its head
+    if (n >= p.N) return;
+    const int hd = p.rope_H * 64;
+    const int region = n / hd, head = (n - region * hd) >> 6; // 0: q, 1: k, 2: v
+    const int half = p.rope_dim >> 1;
+    const bool rotated = region < 2 && d0 < p.rope_dim, low = d0 < half;
+    const int shift = low ? half : -half; // to the partner's columns (where rotated)
+    const half8_t bias = *reinterpret_cast<const half8_t *>(p.bias + n);
+    half8_t biasp = bias;
+    if (rotated) biasp = *reinterpret_cast<const half8_t *>(p.bias + n + shift);
+    half_t *dst0 = (region == 0 ? p.rope_q + size_t(head) * p.M * 64 : (region == 1 ? p.rope_ck : p.rope_cv) + (size_t(head) * p.rope_max_seq + p.rope_pos0) * 64) + d0;
+#pragma unroll
+    for (int r = 0; r < ROWS / 32; r++) {
+        const int ml = r * 32 + (t >> 4), m = m0 + ml;
+        if (m >= p.M) continue;
+        const half8_t v = *reinterpret_cast<const half8_t *>(scratch + ml * TILE_PITCH + nl);
+        half8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] = apply_epilogue_v<MOON_EPI_BIAS>((float)v[e], bias[e]);
+        if (rotated) {
+            const half8_t vp = *reinterpret_cast<const half8_t *>(scratch + ml * TILE_PITCH + nl + shift);
+            const float4 *tab = reinterpret_cast<const float4 *>(p.rope_table + ((size_t)(p.rope_pos0 + m) * half + (low ? d0 : d0 - half)) * 2);
+#pragma unroll
+            for (int e4 = 0; e4 < 4; e4++) {
+                const float4 cs = tab[e4]; // (cos, sin) of two consecutive d
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int e = 2 * e4 + j;
+                    const float c = j ? cs.z : cs.x, sn = j ? cs.w : cs.y;
+                    const half_t mine = o[e], other = apply_epilogue_v<MOON_EPI_BIAS>((float)vp[e], biasp[e]);
+                    half_t a, b;
+                    if (low) {
+                        rotate_pair((float)mine, (float)other, c, sn, a, b);
+                        o[e] = a;
+                    } else {
+                        rotate_pair((float)other, (float)mine, c, sn, a, b);
+                        o[e] = b;
+                    }
+                }
+            }
+        }
+        *reinterpret_cast<half8_t *>(dst0 + size_t(m) * 64) = o;
+    }
+}
+
 // The same tile computation, specialised by wavefront.  A 512-thread workgroup holds four LOADER wavefronts and four
 // MULTIPLIER wavefronts, one of each per SIMD, so the hardware interleaves their instruction streams:
 //   * loaders copy the operand tiles global -> LDS with buffer_load_dwordx4 ... lds (every lane names a 16-byte source,
@@ -512,12 +564,14 @@ template <int MI> struct Dma2 {
 
 // PARTIAL: the workgroup multiplies k-tiles [kt0, kt0 + n_ktiles) of tile `wg` only and leaves the f32 sums in slab `split` of
 // p.partial (no epilogue); otherwise the whole of K, and wg is taken from the workgroup index.
-template <int EPI, int MI, bool PARTIAL = false>
+// ROPE: the epilogue of a qkv projection that writes the rotated q and the cache rows (gemm_tile_out_rope) instead of C.
+template <int EPI, int MI, bool PARTIAL = false, bool ROPE = false>
 __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p, int wg_arg = 0, int kt0 = 0, int n_ktiles_arg = 0, int split = 0) {
     static_assert(MI == 3 || MI == 4, "192- or 256-row tiles");
     static_assert(!PARTIAL || EPI == MOON_EPI_NONE, "partial sums take no epilogue");
+    static_assert(!ROPE || (EPI == MOON_EPI_BIAS && !PARTIAL), "the rotating epilogue follows a bias");
     constexpr int BM2 = Dma2<MI>::BM2, STAGE2_HALFS = Dma2<MI>::STAGE2_HALFS, A_LOADS = Dma2<MI>::A_LOADS;
-    constexpr bool SHARED_EPILOGUE = EPI == MOON_EPI_BIAS_GELU && !PARTIAL; // all eight wavefronts finish the tile
+    constexpr bool SHARED_EPILOGUE = (EPI == MOON_EPI_BIAS_GELU || ROPE) && !PARTIAL; // all eight wavefronts finish the tile
     static_assert(size_t(BM2) * TILE_PITCH <= size_t(DMA2_STAGES) * STAGE2_HALFS, "the parked tile fits the staging area");
     extern __shared__ __attribute__((aligned(16))) half_t lds2[]; // [stage][act: 256 rows | weight: 128 rows][64 halfs]
 
@@ -584,7 +638,8 @@ __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p, int wg_arg 
         if constexpr (SHARED_EPILOGUE) { // the loaders take their half of the epilogue (see the multipliers' end)
             lds_barrier();               // the multipliers have read the last k-tile
             lds_barrier();               // ... and parked the tile
-            gemm_tile_out<EPI, BM2>(p, m0, n0, t, lds2);
+            if constexpr (ROPE) gemm_tile_out_rope<BM2>(p, m0, n0, t, lds2);
+            else gemm_tile_out<EPI, BM2>(p, m0, n0, t, lds2);
         }
         return;
     }
@@ -686,7 +741,8 @@ __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p, int wg_arg 
                     *reinterpret_cast<half4_t *>(lds2 + (wm * 32 * MI + mi * 32 + frag_row) * TILE_PITCH + wn * 64 + ni * 32 + 8 * q + 4 * frag_g) = o;
                 }
         lds_barrier();
-        gemm_tile_out<EPI, BM2>(p, m0, n0, t, lds2);
+        if constexpr (ROPE) gemm_tile_out_rope<BM2>(p, m0, n0, t, lds2);
+        else gemm_tile_out<EPI, BM2>(p, m0, n0, t, lds2);
         return;
     }
     if constexpr (PARTIAL) {
@@ -749,6 +805,14 @@ __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma256_kernel(GemmArgs p)
 template <int EPI>
 __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma192_kernel(GemmArgs p) {
     gemm_nt_dma2_body<EPI, 3>(p);
+}
+
+// A decoder block's qkv projection with the rotation and the cache update in its epilogue (one kernel per tile height)
+__global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma256_rope_kernel(GemmArgs p) {
+    gemm_nt_dma2_body<MOON_EPI_BIAS, 4, false, true>(p);
+}
+__global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma192_rope_kernel(GemmArgs p) {
+    gemm_nt_dma2_body<MOON_EPI_BIAS, 3, false, true>(p);
 }
 
 // TWO products with the same [M, N] result shape in one launch, each with its own split of K, f32 partial sums only (the
@@ -1214,6 +1278,65 @@ int launch_gemm_partials(moon_ctx *ctx, const half_t *A, const half_t *B, size_t
         return MOON_OK;
     }
     return rc;
+}
+
+int launch_gemm_qkv_rope(moon_ctx *ctx, const half_t *A, const half_t *W, const half_t *bias, size_t M, size_t K, half_t *q_out, half_t *cache_k,
+                         half_t *cache_v, const float *table, size_t H, size_t D, size_t rot_dim, size_t max_seq, size_t pos0, bool *done) {
+    *done = false;
+    const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    const size_t N = 3 * H * D, buf_max = (size_t(1) << 31) - 4096;
+    const auto al16 = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+    if (ctx->gemm_kernel[0] || getenv("MOON_GEMM_NO_ROPE")) return MOON_OK; // (a kernel was named for measurements, or the fusion switched off)
+    if (D != 64 || !H || rot_dim % 16 || rot_dim > D || !M || M > 0x3fffffff || K % BK || !K || pos0 + M > max_seq || max_seq > 0x3fffffff) return MOON_OK;
+    if (M * K * 2 >= buf_max || N * K * 2 >= buf_max) return MOON_OK;
+    if (!al16(A) || !al16(W) || !al16(bias) || !al16(q_out) || !al16(cache_k) || !al16(cache_v) || !al16(table)) return MOON_OK;
+    // the shapes that launch_gemm gives to the 256- and 192-row kernels: more 128 x 128 tiles than compute units
+    const int tiles_n = (int)((N + BN - 1) / BN);
+    if (size_t((M + BM - 1) / BM) * tiles_n <= size_t(cus)) return MOON_OK;
+    const int t256 = (int)((M + 255) / 256) * tiles_n, t192 = (int)((M + 191) / 192) * tiles_n;
+    const bool use192 = t192 <= cus && t192 > t256 && ((M + 191) / 192) * 192 <= ((M + 255) / 256) * 256;
+    GemmArgs p;
+    p.A = A;
+    p.Bt = W;
+    p.bias = bias;
+    p.resid = nullptr;
+    p.C = nullptr;
+    p.partial = nullptr;
+    p.M = (int)M;
+    p.N = (int)N;
+    p.K = (int)K;
+    p.tiles_m = (int)(use192 ? (M + 191) / 192 : (M + 255) / 256);
+    p.tiles_n = tiles_n;
+    p.splits = 1;
+    p.k_per_split = (int)K;
+    p.a_bytes = (int)(M * K * 2);
+    p.bt_bytes = (int)(N * K * 2);
+    p.lds_epilogue = 1;
+    p.super_m = p.super_n = 1;
+    p.rope_q = q_out;
+    p.rope_ck = cache_k;
+    p.rope_cv = cache_v;
+    p.rope_table = table;
+    p.rope_H = (int)H;
+    p.rope_dim = (int)rot_dim;
+    p.rope_max_seq = (int)max_seq;
+    p.rope_pos0 = (int)pos0;
+    const int total = p.tiles_m * p.tiles_n;
+    const size_t lds_bytes = use192 ? Dma2<3>::LDS_BYTES : Dma2<4>::LDS_BYTES;
+    static std::atomic<bool> attr_set[2][64];
+    const int dev = ctx->device >= 0 && ctx->device < 64 ? ctx->device : -1;
+    if (dev < 0 || !attr_set[use192 ? 1 : 0][dev].load()) {
+        const void *kern = use192 ? reinterpret_cast<const void *>(gemm_nt_dma192_rope_kernel) : reinterpret_cast<const void *>(gemm_nt_dma256_rope_kernel);
+        MOON_HIP(ctx, hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        if (dev >= 0) attr_set[use192 ? 1 : 0][dev].store(true);
+    }
+    const dim3 grid(((total + 7) / 8) * 8);
+    if (use192) hipLaunchKernelGGL(gemm_nt_dma192_rope_kernel, grid, dim3(DMA_THREADS), lds_bytes, ctx->stream, p);
+    else hipLaunchKernelGGL(gemm_nt_dma256_rope_kernel, grid, dim3(DMA_THREADS), lds_bytes, ctx->stream, p);
+    MOON_NOTE_KERNEL(ctx, "%s %d workgroups", use192 ? "gemm_nt_dma192_rope_kernel" : "gemm_nt_dma256_rope_kernel", total);
+    MOON_HIP(ctx, hipGetLastError());
+    *done = true;
+    return MOON_OK;
 }
 
 int launch_gemm_pair_ln(moon_ctx *ctx, const half_t *A_add, const half_t *B_add, const half_t *bias_add, size_t K_add, const half_t *A, const half_t *B,

@@ -23,6 +23,11 @@ struct GemmArgs {
     int a_bytes, bt_bytes; // sizes of A and Bt (the wavefront-specialised kernels address them as buffers; < 2^31)
     int lds_epilogue; // write the tile through LDS in full lines (needs 16-byte aligned C / bias / resid rows)
     int super_m, super_n; // gemm_wide.hpp: tiles are dealt in blocks of super_m x super_n tiles (>= 1 each)
+    // the *_rope kernels only: the product is a decoder block's qkv projection [M, 3 * H * 64]; instead of C they write the
+    // rotated q [H][M][64] and the cache rows [H][max_seq][64] of k (rotated) and v at positions pos0 .. pos0 + M - 1
+    half_t *rope_q, *rope_ck, *rope_cv;
+    const float *rope_table; // [max_seq][rot_dim / 2][2] (cos, sin)
+    int rope_H, rope_dim, rope_max_seq, rope_pos0;
 };
 
 template <int N>

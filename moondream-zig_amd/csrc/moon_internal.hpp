@@ -124,6 +124,12 @@ int launch_gemm_partials(moon_ctx *ctx, const half_t *A, const half_t *B, size_t
                          int *splits);
 int launch_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias, half_t *C,
                 size_t M, size_t N, size_t K, int b_layout, int epilogue, const half_t *resid = nullptr, const GemmLayerNorm *ln = nullptr);
+// A decoder block's qkv projection [M, K] . [3 * H * D, K]^T + bias with launch_qkv_rope_cache folded into its epilogue: the
+// rotated q goes to q_out [H][M][D], the rotated k and v to rows pos0 .. pos0 + M - 1 of the cache [H][max_seq][D]; the
+// projection itself is not written anywhere.  The same bits as the two launches.  Only for D = 64 and the shapes that take the
+// 256- or 192-row product kernels; *done says whether anything was launched.
+int launch_gemm_qkv_rope(moon_ctx *ctx, const half_t *A, const half_t *W, const half_t *bias, size_t M, size_t K, half_t *q_out, half_t *cache_k,
+                         half_t *cache_v, const float *table, size_t H, size_t D, size_t rot_dim, size_t max_seq, size_t pos0, bool *done);
 // Two products with the same [M, N] result in ONE launch, then the launch that finishes both, as launch_gemm does with
 // ln->add_partial set: C = f16(resid + f16(add + t)), add = f16(f16(A_add . B_add^T) + bias_add), t = f16(f16(A . B^T) + bias),
 // and the LayerNorm of the finished rows into ln.out (ln.add must name M x N halfs all the same).  Both B operands are [N, K].

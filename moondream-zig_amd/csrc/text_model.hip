@@ -307,8 +307,12 @@ int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool p
         MOON_TRY(launch_gemv_nt(ctx, m->ln_in, fc1_w, fc1_b, m->fc1, z.ffn, z.d, MOON_EPI_BIAS_GELU));
         MOON_TRY(launch_gemv_nt(ctx, m->fc1, fc2_w, fc2_b, m->mlp, z.d, z.ffn, MOON_EPI_BIAS));
     } else {
-        MOON_TRY(launch_gemm(ctx, m->ln_in, qkv_w, qkv_b, m->qkv, n, 3 * z.d, z.d, MOON_B_NK, MOON_EPI_BIAS));
-        MOON_TRY(launch_qkv_rope_cache(ctx, m->qkv, m->q_rot, ck, cv, m->freqs, n, z.H, z.D, m->cfg.rot_dim, z.S, pos));
+        bool roped = false; // the projection with the rotation and the cache update in its epilogue, where the shape has that form
+        MOON_TRY(launch_gemm_qkv_rope(ctx, m->ln_in, qkv_w, qkv_b, n, z.d, m->q_rot, ck, cv, m->freqs, z.H, z.D, m->cfg.rot_dim, z.S, pos, &roped));
+        if (!roped) {
+            MOON_TRY(launch_gemm(ctx, m->ln_in, qkv_w, qkv_b, m->qkv, n, 3 * z.d, z.d, MOON_B_NK, MOON_EPI_BIAS));
+            MOON_TRY(launch_qkv_rope_cache(ctx, m->qkv, m->q_rot, ck, cv, m->freqs, n, z.H, z.D, m->cfg.rot_dim, z.S, pos));
+        }
         MOON_TRY(launch_sdpa(ctx, m->q_rot, ck, cv, m->attn, z.H, n, pos + n, z.D, z.S * z.D, (long)pos, nullptr, 0, true));
         const bool finish_in_fc2 = chain_ln && layer + 1 < z.L;
         if (finish_in_fc2) {

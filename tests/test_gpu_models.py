@@ -261,6 +261,35 @@ def test_prefill_with_out_proj_and_fc2_in_one_launch(moon, O, ctx, monkeypatch):
     assert max(errs) <= TOL
 
 
+def test_prefill_with_the_rotation_in_the_qkv_product(moon, O, ctx, monkeypatch):
+    """Where the qkv projection takes the 192- / 256-row kernels its epilogue rotates q and k and writes the cache rows
+    itself; MOON_GEMM_NO_ROPE runs the projection and the rotation as two launches.  The same values, roundings and
+    rotations: hidden states, logits and the ids decoded from the cache are the same bits, for a ragged first chunk at
+    position 0 and a second chunk that starts at position 333."""
+    cfg = dict(O.TEXT_CFG, n_layers=2, vocab=2048)
+    ref, dev = _text_pair(moon, O, ctx, cfg, seed=5)
+    a, b = O.fill_uniform_u32(333, 0, 52, cfg["vocab"]), O.fill_uniform_u32(200, 0, 53, cfg["vocab"])
+    out = []
+    for fused in (True, False):
+        if not fused:
+            monkeypatch.setenv("MOON_GEMM_NO_ROPE", "1")
+        dev.reset()
+        dev.forward(a)
+        h1 = dev.hidden(333).copy()
+        dev.forward(b)
+        h2, lg = dev.hidden(200).copy(), dev.logits().copy()
+        out.append((h1, h2, lg, dev.greedy(6).tolist()))
+    monkeypatch.delenv("MOON_GEMM_NO_ROPE")
+    dev.close()
+    for x, y in zip(out[0][:3], out[1][:3]):
+        assert np.array_equal(x.view(np.uint16), y.view(np.uint16))
+    assert out[0][3] == out[1][3]
+    cache = ref.new_cache()
+    ref.text_decoder(ref.text_encoder(a), cache)
+    h_ref = ref.text_decoder(ref.text_encoder(b), cache)
+    assert O.rel_frobenius(out[0][1], h_ref) <= TOL
+
+
 def test_sessions_built_from_a_moondream_bin_file(moon, O, ctx, tmp_path):
     """Weights written in the reference's file layout, mapped by the library's reader and uploaded from the mapping: the
     decoder and the vision encoder give the same bits as when built from in-memory arrays, and match the oracle."""
