@@ -314,11 +314,14 @@ int layer_forward(moon_text_model *m, size_t layer, size_t n, size_t pos, bool p
             MOON_TRY(launch_qkv_rope_cache(ctx, m->qkv, m->q_rot, ck, cv, m->freqs, n, z.H, z.D, m->cfg.rot_dim, z.S, pos));
         }
         MOON_TRY(launch_sdpa(ctx, m->q_rot, ck, cv, m->attn, z.H, n, pos + n, z.D, z.S * z.D, (long)pos, nullptr, 0, true));
-        const bool finish_in_fc2 = chain_ln && layer + 1 < z.L;
+        const bool finish_in_fc2 = chain_ln;
         if (finish_in_fc2) {
             // out_proj and fc2 as one launch (each alone leaves a quarter of the device idle at 768 rows), finished together
+            // with the LayerNorm that comes next: the next block's, or after the last block the model's final one (which the
+            // LM head applies to the one row it needs by itself; here it only keeps the last block on the same launches)
             MOON_TRY(launch_gemm(ctx, m->ln_in, fc1_w, fc1_b, m->fc1, n, z.ffn, z.d, MOON_B_NK, MOON_EPI_BIAS_GELU));
-            GemmLayerNorm next{m->ln_w + (layer + 1) * z.d, m->ln_b + (layer + 1) * z.d, m->ln_in, m->cfg.ln_eps};
+            const bool last = layer + 1 == z.L;
+            GemmLayerNorm next{last ? m->lno_w : m->ln_w + (layer + 1) * z.d, last ? m->lno_b : m->ln_b + (layer + 1) * z.d, m->ln_in, m->cfg.ln_eps};
             next.add = m->attn_proj;
             next.add_scratch = m->mlp;
             bool done = false;
