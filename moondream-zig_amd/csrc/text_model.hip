@@ -7,6 +7,7 @@
 #include "moon_internal.hpp"
 
 #include <cstdlib>
+#include <cstring>
 #include <algorithm>
 #include <vector>
 
@@ -65,6 +66,7 @@ struct moon_text_model {
     half_t *hidden = nullptr, *ln_in = nullptr, *qkv = nullptr, *q_rot = nullptr, *attn = nullptr, *attn_proj = nullptr,
            *fc1 = nullptr, *mlp = nullptr, *logits = nullptr, *ln_last = nullptr;
     uint32_t *ids_dev = nullptr;   // [max_seq] prompt ids / generated ids
+    uint32_t *ids_pinned = nullptr; // [max_seq] page-locked host memory the prompt ids are copied from (a copy from pageable memory blocks the call)
     float *u_dev = nullptr;        // [max_seq] the sampling loop's random numbers, one per step
     uint32_t *state_dev = nullptr; // [0] position (KV length), [1] tokens recorded, [2] current token, [3] stopped, [4] eos id + 1 (record_token)
     size_t cur_len = 0, last_n = 0;
@@ -162,6 +164,7 @@ int alloc_all(moon_text_model *m) {
     MOON_TRY(dalloc_t(m, z.V, &m->logits));
     MOON_TRY(dalloc_t(m, z.d, &m->ln_last));
     MOON_TRY(dalloc_t(m, z.S, &m->ids_dev));
+    MOON_HIP(m->ctx, hipHostMalloc((void **)&m->ids_pinned, z.S * sizeof(uint32_t), hipHostMallocDefault));
     MOON_TRY(dalloc_t(m, z.S, &m->u_dev));
     MOON_TRY(dalloc_t(m, 8, &m->state_dev));
     MOON_TRY(launch_fill_uniform_u32(m->ctx, m->state_dev, 8, 0, 0, 1)); // zeros
@@ -198,6 +201,8 @@ void free_all(moon_text_model *m) {
     (void)hipStreamSynchronize(m->ctx->stream);
     for (void *p : m->allocs) (void)hipFree(p);
     m->allocs.clear();
+    if (m->ids_pinned) (void)hipHostFree(m->ids_pinned);
+    m->ids_pinned = nullptr;
 }
 
 // Counters, exchange buffers and error words of the fused decode kernels back to their initial state (fill kernels in
@@ -532,7 +537,8 @@ extern "C" int moon_text_forward(moon_text_model *m, const uint32_t *ids, size_t
     for (size_t i = 0; i < n_ids; i++)
         if (ids[i] >= m->cfg.vocab) return moon_fail(ctx, MOON_ETOKEN, "text_forward: token id %u >= vocab %zu (TokenIdOutOfBounds)", ids[i], m->cfg.vocab);
     MOON_HIP(ctx, hipSetDevice(ctx->device));
-    MOON_HIP(ctx, hipMemcpyAsync(m->ids_dev, ids, n_ids * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
+    memcpy(m->ids_pinned, ids, n_ids * sizeof(uint32_t)); // (every call ends with the stream drained: the buffer is free)
+    MOON_HIP(ctx, hipMemcpyAsync(m->ids_dev, m->ids_pinned, n_ids * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
     MOON_TRY(launch_embed(ctx, m->wte, m->ids_dev, m->hidden, n_ids, m->cfg.dim));
     return forward_rows_locked(m, n_ids);
 }
