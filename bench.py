@@ -109,7 +109,7 @@ def bench_decoder(moon, ctx, steps, warmup, decode_mode=None):
     t0 = time.perf_counter()
     model.forward(ids)
     ctx.sync()
-    prefill_s = time.perf_counter() - t0
+    prefill_samples = [time.perf_counter() - t0]
     # The timed region: exactly `steps` decoded tokens after `warmup` untimed ones, from the same cache length every time.
     # One such sample is only 10-15 ms long, so it is repeated REPEATS times (prefill again, warm up again, time the same
     # steps) and the median is reported; every repeat's figure is kept in the output.
@@ -117,7 +117,11 @@ def bench_decoder(moon, ctx, steps, warmup, decode_mode=None):
     for rep in range(REPEATS):
         if rep:
             model.reset()
+            ctx.sync()
+            t0 = time.perf_counter()
             model.forward(ids)
+            ctx.sync()
+            prefill_samples.append(time.perf_counter() - t0)
         if warmup:
             model.greedy(warmup)
         ctx.sync()
@@ -127,10 +131,11 @@ def bench_decoder(moon, ctx, steps, warmup, decode_mode=None):
         ctx.sync()
         samples.append(time.perf_counter() - t0)
     dt = sorted(samples)[len(samples) // 2]
+    prefill_s = sorted(prefill_samples)[len(prefill_samples) // 2]  # (the first call of the session is reported apart)
     wbytes = model.weight_bytes_per_token
     # K and V of every layer are read once per token: 2 * L * H * HD * 2 bytes per cached position
     kv_bytes = sum(2 * L * H * HD * 2 * (kv0 + s + 1) for s in range(steps)) / steps
-    res = dict(tokens_per_s=steps / dt, ms_per_token=dt / steps * 1e3, prefill_tokens=PREFILL, prefill_ms=prefill_s * 1e3, prefill_first_call_ms=prefill_first_s * 1e3,
+    res = dict(tokens_per_s=steps / dt, ms_per_token=dt / steps * 1e3, prefill_tokens=PREFILL, prefill_ms=prefill_s * 1e3, prefill_repeats_ms=[x * 1e3 for x in prefill_samples], prefill_first_call_ms=prefill_first_s * 1e3,
                setup_s=setup_s, kv_len_start=kv0, weight_bytes_per_token=wbytes, kv_bytes_per_token=kv_bytes,
                hbm_gbs=(wbytes + kv_bytes) / (dt / steps) / 1e9, first_tokens=toks[:8].tolist(),
                repeats_ms_per_token=[x / steps * 1e3 for x in samples], reported="median of the repeats")
