@@ -324,6 +324,51 @@ def test_sessions_built_from_a_moondream_bin_file(moon, O, ctx, tmp_path):
     vis_file.close()
 
 
+@pytest.mark.timeout(900)
+def test_full_size_moondream_bin_round_trip(moon, O, ctx, tmp_path):
+    """A moondream.bin with all 36 tensors at the reference's sizes (weights.zig:397-523; 3.7 GB, offsets past 2^32),
+    written in the reference's layout, mapped by the library's reader and uploaded from the mapping.  The decoder built from
+    the file gives the same bits as the decoder whose weights the device generator made from the same seed (so every text
+    tensor is found, has the expected shape and lands in its place), and the vision session with its patch embedding and
+    projection the same bits as the one built from the in-memory arrays."""
+    tcfg, vcfg, io = O.TEXT_CFG, O.VISION_CFG, O.VISION_IO_CFG
+    tw = O.synth_text_weights(tcfg, 0)
+    vw, iw = O.synth_vision_weights(vcfg, 0), O.synth_vision_io_weights(vcfg, io, 0)
+    tensors = O.text_bin_tensors(tw)
+    tensors.update(O.vision_bin_tensors(vw))
+    tensors.update({"v_" + k: v for k, v in iw.items()})
+    assert len(tensors) == 36
+    path = str(tmp_path / "moondream.bin")
+    O.write_moondream_bin(path, tensors)
+    import os
+    size = os.path.getsize(path)
+    assert size > 3_600_000_000 and size == 8 + sum(12 + len(k) + 8 * v.ndim + 2 * v.size for k, v in tensors.items())
+    del tensors, tw
+    mvcfg = moon.vision_model.make_config(**vcfg)
+    with moon.weights.BinFile(path) as f:
+        assert len(f) == 36
+        txt = moon.text_model.TextModel(moon.text_model.default_config(), weights=f, ctx=ctx)
+        vis = moon.vision_model.VisionModel(mvcfg, weights=f, ctx=ctx)
+        vis.attach_io(weights=f)
+    os.remove(path)  # the mapping is closed: the sessions own device copies
+    gen = moon.text_model.TextModel(moon.text_model.default_config(), seed=0, std=0.02, ctx=ctx)
+    ids = O.fill_uniform_u32(40, 0, 54, tcfg["vocab"])
+    out = []
+    for dev in (txt, gen):
+        dev.forward(ids)
+        out.append((dev.hidden(40).copy(), dev.logits().copy(), dev.greedy(4).tolist()))
+        dev.close()
+    assert np.array_equal(out[0][0].view(np.uint16), out[1][0].view(np.uint16))
+    assert np.array_equal(out[0][1].view(np.uint16), out[1][1].view(np.uint16)) and out[0][2] == out[1][2]
+    mem = moon.vision_model.VisionModel(mvcfg, weights=vw, ctx=ctx)
+    mem.attach_io(weights=iw)
+    patches = O.fill_normal_f16((2 * io["tokens"], io["patch_dim"]), 0, 302, 1.0)
+    a, b = vis.encode_image(patches), mem.encode_image(patches)
+    assert np.isfinite(a.astype(np.float32)).all() and np.array_equal(a.view(np.uint16), b.view(np.uint16))
+    vis.close()
+    mem.close()
+
+
 @pytest.mark.parametrize("case", ["ties", "nan_at_0", "nan_elsewhere", "all_neg_inf", "max_is_last"])
 def test_greedy_argmax_rules_in_every_mode(moon, O, ctx, case):
     """The greedy loop's arg-max (fused into the LM-head launch)
