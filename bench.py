@@ -373,18 +373,21 @@ def bench_gemv(moon, ctx, iters=256):
                                            frac=N * K * 2 / us_read / 1e3 / HBM_PEAK_GBS))
 
 
-def bench_gemm(moon, ctx, M, K, N, iters=50):
+def bench_gemm(moon, ctx, M, K, N, iters=50, b_kn=False):
+    """b_kn: the second operand as hgemm.zig takes it, [K, N]; otherwise the resident form [N, K] (the sessions transpose the
+    vision weights once at load time)."""
     L_ = moon._lib
     a = ctx.alloc(M * K * 2)
     a.fill_normal(M * K, 0, 0, 1.0)
-    wt = ctx.alloc(N * K * 2)  # resident form [N,K] (vision weights are transposed once at load time)
+    wt = ctx.alloc(N * K * 2)
     wt.fill_normal(N * K, 0, 1, 0.02)
     b = ctx.alloc(N * 2)
     b.fill_normal(N, 0, 2, 0.02)
     c = ctx.alloc(M * N * 2)
+    layout = L_.B_KN if b_kn else L_.B_NK
 
     def launch(i):
-        ctx.check(ctx.lib.moon_dev_linear(ctx.handle, a.ptr, M, K, wt.ptr, N, L_.B_NK, b.ptr, L_.EPI_BIAS, c.ptr))
+        ctx.check(ctx.lib.moon_dev_linear(ctx.handle, a.ptr, M, K, wt.ptr, N, layout, b.ptr, L_.EPI_BIAS, c.ptr))
 
     us, us_ev = launch_time_us(ctx, launch, iters)
     kernel = ctx.last_kernel()
@@ -567,6 +570,8 @@ def main():
         calibration_copies(ctx)
     if args.only_gemm:
         out = {"gemm_vision_fc1": bench_gemm(moon, ctx, 729, 1152, 4304), "gemm_vision_fc2": bench_gemm(moon, ctx, 729, 4304, 1152),
+               "gemm_vision_fc1_kn_operand": bench_gemm(moon, ctx, 729, 1152, 4304, b_kn=True),
+               "gemm_vision_fc2_kn_operand": bench_gemm(moon, ctx, 729, 4304, 1152, b_kn=True),
                "gemm_vision_qkv": bench_gemm(moon, ctx, 729, 1152, 3456), "gemm_vision_fc1_m1458": bench_gemm(moon, ctx, 1458, 1152, 4304),
                "gemm_prefill_fc1": bench_gemm(moon, ctx, 768, 2048, 8192), "gemm_prefill_fc2": bench_gemm(moon, ctx, 768, 8192, 2048),
                "gemm_4096": bench_gemm(moon, ctx, 4096, 4096, 4096, iters=20), "attention": bench_attention(moon, ctx),
@@ -597,6 +602,7 @@ def main():
         extra["op_level_decode_registered_weights"] = bench_op_level_decode(moon, ctx)
         extra["gemm_vision_fc1"] = bench_gemm(moon, ctx, 729, 1152, 4304)
         extra["gemm_vision_fc2"] = bench_gemm(moon, ctx, 729, 4304, 1152)
+        extra["gemm_vision_fc1_kn_operand"] = bench_gemm(moon, ctx, 729, 1152, 4304, b_kn=True)  # hgemm.zig's own operand layout
         extra["gemm_vision_fc1_m1458"] = bench_gemm(moon, ctx, 1458, 1152, 4304)
         extra["attention"] = bench_attention(moon, ctx)
         extra["vision_encoder_27_blocks"] = bench_vision(moon, ctx)

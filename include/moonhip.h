@@ -436,6 +436,8 @@ int moon_bin_vision_io_weights(const moon_bin *bin, const moon_vision_config *cf
  *   MOON_GEMM_NO_PAIR=1            text prefill: a block's out_proj and fc2 run as launches of their own instead of one joint launch
  *                                  (read at every call); the two forms split K differently, so their f32 sums, and with them a few
  *                                  f16 roundings, differ
+ *   MOON_GEMM_KN_TRANSPOSE=1       products with a [K, N] second operand always run over a transposed copy instead of reading the operand
+ *                                  in place where the shape allows (read at every call; the same bits either way)
  *   MOON_GEMM_NO_ROPE=1            text prefill: the qkv projection and the rotation + cache update run as two launches instead of
  *                                  one (read at every call; the same bits either way)
  * Every other setting gives the same results, bit for bit; only the time changes. */

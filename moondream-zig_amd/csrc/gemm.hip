@@ -350,7 +350,12 @@ constexpr int DMA_STAGES = 4;
 constexpr int DMA_THREADS = 512;
 constexpr size_t DMA_LDS_BYTES = size_t(DMA_STAGES) * 2 * TILE_HALFS * sizeof(half_t);
 
-template <int EPI>
+// BKN: the second operand is [K, N] (hgemm.zig's layout) and is read as it lies.  Its tile sits in LDS as [k][128 n]; a
+// loader instruction copies four k-rows of 256 bytes, the 16-byte granules of row r XOR-ed with 2 * (r & 3) on the source
+// side, and the multipliers fetch their operand slices with the transposing LDS load (ds_read_b64_tr_b16: the 16 lanes of a
+// quarter-wavefront name a 4 x 16 block, four halfs each, and lane i receives column i of its four rows), two per slice in
+// place of one 16-byte read.  Same products in the same order as with the [N, K] operand: the same bits.  Needs N % 8 == 0.
+template <int EPI, bool BKN = false>
 __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma_kernel(GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) half_t lds_dma[]; // [stage][operand: 0 = act (m), 1 = weight (n)][TILE_HALFS]
 
@@ -386,16 +391,21 @@ __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma_kernel(GemmArgs p) {
             const int g8 = swz(r, lane & 7) * 8;
             off_a[j] = (min(m0 + r, p.M - 1) * p.K + g8) * 2;
             off_w[j] = (min(n0 + r, p.N - 1) * p.K + g8) * 2;
+            if (BKN) { // k-rows 16 * role_wave + 4 * j .. + 3 of the tile: lane -> (row, physical granule); columns past N are never stored
+                const int rk = 16 * role_wave + 4 * j + (lane >> 4), pg = lane & 15;
+                off_w[j] = (rk * p.N + n0 + (pg ^ (2 * (rk & 3))) * 8) * 2;
+            }
         }
         auto issue = [&](int kt) {
             half_t *stage = lds_dma + size_t(kt % DMA_STAGES) * 2 * TILE_HALFS;
             // the k-tile enters through the descriptors' base and size: the range check that turns reads past the end of the
             // operand into zeros does not see an instruction's scalar offset
             const int k_off = (k_begin + kt * BK) * 2;
+            const int kw_off = BKN ? (k_begin + kt * BK) * p.N * 2 : k_off; // (rows of [K, N] past K lie past the end: zeros)
             const __amdgpu_buffer_rsrc_t rs_a =
                 __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(reinterpret_cast<const char *>(p.A)) + k_off, 0, p.a_bytes - k_off, 0x00020000);
             const __amdgpu_buffer_rsrc_t rs_w =
-                __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(reinterpret_cast<const char *>(p.Bt)) + k_off, 0, p.bt_bytes - k_off, 0x00020000);
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(reinterpret_cast<const char *>(p.Bt)) + kw_off, 0, p.bt_bytes - kw_off, 0x00020000);
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (__attribute__((address_space(3))) void *)(stage + (32 * role_wave + 8 * j) * BK), 16,
@@ -455,39 +465,64 @@ __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma_kernel(GemmArgs p) {
             off_a[s][i] = (rm * BK + swz(rm, 2 * s + frag_g) * 8) * 2;
             off_w[s][i] = (TILE_HALFS + rn * BK + swz(rn, 2 * s + frag_g) * 8) * 2;
         }
+    // BKN: where this lane points the transposing loads of n-block ni, for the first four k of its slice of step 0 (step s and
+    // the second four add (16 s + 4 q) rows of 256 bytes): row 8 * frag_g + i / 4, columns 4 * (i % 4) .. + 3 of the 16 the
+    // lane's quarter-wavefront covers, i = lane % 16
+    unsigned off_wk[2];
+#pragma unroll
+    for (int ni = 0; ni < 2; ni++) {
+        const int i = lane & 15, row = 8 * frag_g + (i >> 2);
+        const int c = wn * 8 + ni * 4 + ((lane >> 4) & 1) * 2 + ((i & 3) >> 1); // 16-byte granule of the row
+        off_wk[ni] = (TILE_HALFS + row * BN + (c ^ (2 * (row & 3))) * 8 + (i & 1) * 4) * 2;
+    }
     // The operand reads and the waits for them are written out by hand.  Left to the compiler the reads sink below the
     // MFMAs of the step before (into the registers those just consumed) and are waited for at once, and the wait at the
     // head of the loop is for everything outstanding, so the LDS latency is paid several times per k-tile with the matrix
     // core idle.  The compiler does not count reads issued from asm statements, so it adds no waits of its own for them;
     // each wait statement names the registers it guards as operands, which keeps their use behind it.
     constexpr unsigned STAGE_BYTES = 2 * TILE_HALFS * sizeof(half_t);
-    auto read_frags = [&](int kt, int s, half8_t (&fa)[2], half8_t (&fw)[2]) {
+    // (BKN: fw[ni] arrives as two 8-byte halves, wk[ni][0..1])
+    struct Frag {
+        half8_t fa[2], fw[2];
+        half4_t wk[2][2];
+    };
+    auto read_frags = [&](int kt, int s, Frag &f) {
         const unsigned sb = unsigned(kt % DMA_STAGES) * STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            asm volatile("ds_read_b128 %0, %1" : "=v"(fa[i]) : "v"(sb + off_a[s][i]));
-            asm volatile("ds_read_b128 %0, %1" : "=v"(fw[i]) : "v"(sb + off_w[s][i]));
+            asm volatile("ds_read_b128 %0, %1" : "=v"(f.fa[i]) : "v"(sb + off_a[s][i]));
+            if (!BKN) asm volatile("ds_read_b128 %0, %1" : "=v"(f.fw[i]) : "v"(sb + off_w[s][i]));
+            else {
+#pragma unroll
+                for (int q = 0; q < 2; q++)
+                    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(f.wk[i][q]) : "v"(sb + off_wk[i] + unsigned(16 * s + 4 * q) * (BN * 2)));
+            }
         }
     };
-    // all but the newest four reads (the group issued last) have landed; fa / fw belong to an older group
-    auto wait_older = [&](half8_t (&fa)[2], half8_t (&fw)[2]) {
-        asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fw[0]), "+v"(fw[1])::"memory");
+    // all but the newest group of reads (the one issued last: four reads, six with BKN) have landed; f belongs to an older group
+    auto wait_older = [&](Frag &f) {
+        if (!BKN) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.fw[0]), "+v"(f.fw[1])::"memory");
+        else
+            asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.wk[0][0]), "+v"(f.wk[0][1]), "+v"(f.wk[1][0]), "+v"(f.wk[1][1])::"memory");
     };
-    auto wait_all = [&](half8_t (&fa)[2], half8_t (&fw)[2]) {
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fw[0]), "+v"(fw[1])::"memory");
+    auto wait_all = [&](Frag &f) {
+        if (!BKN) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.fw[0]), "+v"(f.fw[1])::"memory");
+        else
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.wk[0][0]), "+v"(f.wk[0][1]), "+v"(f.wk[1][0]), "+v"(f.wk[1][1])::"memory");
     };
-    auto multiply = [&](const half8_t (&fa)[2], const half8_t (&fw)[2]) {
+    auto multiply = [&](const Frag &f) {
 #pragma unroll
-        for (int ni = 0; ni < 2; ni++)
+        for (int ni = 0; ni < 2; ni++) {
+            const half8_t w = BKN ? __builtin_shufflevector(f.wk[ni][0], f.wk[ni][1], 0, 1, 2, 3, 4, 5, 6, 7) : f.fw[ni];
 #pragma unroll
-            for (int mi = 0; mi < 2; mi++)
-                acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[ni], fa[mi], acc[ni][mi], 0, 0, 0);
+            for (int mi = 0; mi < 2; mi++) acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w, f.fa[mi], acc[ni][mi], 0, 0, 0);
+        }
     };
 
-    half8_t fa[2][2], fw[2][2];
+    Frag fr[2];
     lds_barrier(); // tile 0 is visible
-    read_frags(0, 0, fa[0], fw[0]);
-    // At the top of a k-tile the reads of its first slice into fa[0]/fw[0] are in flight.  Every slice is requested one
+    read_frags(0, 0, fr[0]);
+    // At the top of a k-tile the reads of its first slice into fr[0] are in flight.  Every slice is requested one
     // step (four MFMAs) before it is multiplied; the barrier that publishes tile kt+1 (and hands the buffer of tile kt
     // back to the loaders, hence the wait for this wavefront's last reads of it) is passed with the MFMAs of the third
     // slice queued, and the first slice of tile kt+1 is fetched under the MFMAs of the fourth.
@@ -497,38 +532,38 @@ __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma_kernel(GemmArgs p) {
     // fences keep the MFMAs of a step where they are written: between the reads of the next slice and the wait for it.
     const int last_steps = ((k_end - k_begin) - (n_ktiles - 1) * BK) / 16; // 16-wide steps of the last k-tile (1..4)
     auto first_three = [&](int kt) {
-        read_frags(kt, 1, fa[1], fw[1]);
-        wait_older(fa[0], fw[0]);
-        multiply(fa[0], fw[0]);
+        read_frags(kt, 1, fr[1]);
+        wait_older(fr[0]);
+        multiply(fr[0]);
         __builtin_amdgcn_sched_barrier(0);
-        read_frags(kt, 2, fa[0], fw[0]);
-        wait_older(fa[1], fw[1]);
-        multiply(fa[1], fw[1]);
+        read_frags(kt, 2, fr[0]);
+        wait_older(fr[1]);
+        multiply(fr[1]);
         __builtin_amdgcn_sched_barrier(0);
-        read_frags(kt, 3, fa[1], fw[1]);
-        wait_older(fa[0], fw[0]);
-        multiply(fa[0], fw[0]);
+        read_frags(kt, 3, fr[1]);
+        wait_older(fr[0]);
+        multiply(fr[0]);
         __builtin_amdgcn_sched_barrier(0);
     };
     for (int kt = 0; kt + 1 < n_ktiles; kt++) {
         first_three(kt);
-        wait_all(fa[1], fw[1]);
+        wait_all(fr[1]);
         __builtin_amdgcn_s_barrier();
-        read_frags(kt + 1, 0, fa[0], fw[0]);
-        multiply(fa[1], fw[1]);
+        read_frags(kt + 1, 0, fr[0]);
+        multiply(fr[1]);
         __builtin_amdgcn_sched_barrier(0);
     }
     if (last_steps == BK / 16) {
         first_three(n_ktiles - 1);
-        wait_all(fa[1], fw[1]);
-        multiply(fa[1], fw[1]);
-    } else { // fa[0] / fw[0] will hold its first slice
-        wait_all(fa[0], fw[0]);
-        multiply(fa[0], fw[0]);
+        wait_all(fr[1]);
+        multiply(fr[1]);
+    } else { // fr[0] will hold its first slice
+        wait_all(fr[0]);
+        multiply(fr[0]);
         for (int s = 1; s < last_steps; s++) {
-            read_frags(n_ktiles - 1, s, fa[0], fw[0]);
-            wait_all(fa[0], fw[0]);
-            multiply(fa[0], fw[0]);
+            read_frags(n_ktiles - 1, s, fr[0]);
+            wait_all(fr[0]);
+            multiply(fr[0]);
         }
     }
     if (p.splits == 1 && p.N % 8 == 0 && p.lds_epilogue) {
@@ -1014,7 +1049,12 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
         return MOON_OK;
     }
     const half_t *Bt = B;
-    if (b_layout == MOON_B_KN) {
+    // A [K, N] operand is read as it lies by the 128 x 128 wavefront-specialised kernel where the shape takes that kernel
+    // (at most one tile per compute unit); other shapes get a transposed copy first.  MOON_GEMM_KN_TRANSPOSE: always the copy.
+    const bool native_kn = b_layout == MOON_B_KN && N % 8 == 0 && K % 16 == 0 && size_t(M) * K * 2 < (size_t(1) << 31) - 4096 &&
+                           size_t(N) * K * 2 < (size_t(1) << 31) - 4096 && !ctx->gemm_kernel[0] && !getenv("MOON_GEMM_KN_TRANSPOSE") &&
+                           size_t((M + BM - 1) / BM) * ((N + BN - 1) / BN) <= size_t(ctx->cu_count > 0 ? ctx->cu_count : 256);
+    if (b_layout == MOON_B_KN && !native_kn) {
         MOON_TRY(moon_grow(ctx, ctx->work[2], size_t(N) * K * sizeof(half_t)));
         hipLaunchKernelGGL(transpose_kernel, dim3((N + 63) / 64, (K + 63) / 64), dim3(256), 0, ctx->stream, B,
                            (half_t *)ctx->work[2].ptr, K, N);
@@ -1183,19 +1223,21 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     bool use_dma = K % 16 == 0 && total <= cus && buffers_ok;
     if (force && !strcmp(force, "regs")) use_dma = false;
     if (force && !strcmp(force, "dma")) use_dma = K % 16 == 0 && buffers_ok;
+    if (native_kn && !use_dma) return moon_fail(ctx, MOON_EINVAL, "gemm: no kernel for this [K, N] operand"); // (cannot happen: the same conditions)
     if (use_dma) {
-        static std::atomic<bool> attr_set[64]; // 128 KiB of dynamic LDS needs the opt-in once per device (and per instantiation)
+        static std::atomic<bool> attr_set[2][64]; // 128 KiB of dynamic LDS needs the opt-in once per device (and per instantiation)
         const int dev = ctx->device >= 0 && ctx->device < 64 ? ctx->device : -1;
-        if (dev < 0 || !attr_set[dev].load()) {
-            MOON_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_nt_dma_kernel<EPI>),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)DMA_LDS_BYTES));
-            if (dev >= 0) attr_set[dev].store(true);
+        if (dev < 0 || !attr_set[native_kn ? 1 : 0][dev].load()) {
+            const void *kern = native_kn ? reinterpret_cast<const void *>(gemm_nt_dma_kernel<EPI, true>) : reinterpret_cast<const void *>(gemm_nt_dma_kernel<EPI>);
+            MOON_HIP(ctx, hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)DMA_LDS_BYTES));
+            if (dev >= 0) attr_set[native_kn ? 1 : 0][dev].store(true);
         }
-        hipLaunchKernelGGL(gemm_nt_dma_kernel<EPI>, dim3(grid), dim3(DMA_THREADS), DMA_LDS_BYTES, ctx->stream, p);
+        if (native_kn) hipLaunchKernelGGL((gemm_nt_dma_kernel<EPI, true>), dim3(grid), dim3(DMA_THREADS), DMA_LDS_BYTES, ctx->stream, p);
+        else hipLaunchKernelGGL(gemm_nt_dma_kernel<EPI>, dim3(grid), dim3(DMA_THREADS), DMA_LDS_BYTES, ctx->stream, p);
     } else {
         hipLaunchKernelGGL(gemm_nt_mfma_kernel<EPI>, dim3(grid), dim3(256), 0, ctx->stream, p);
     }
-    MOON_NOTE_KERNEL(ctx, "%s %d workgroups, k split %d%s", use_dma ? "gemm_nt_dma_kernel" : "gemm_nt_mfma_kernel", total, splits,
+    MOON_NOTE_KERNEL(ctx, "%s %d workgroups, k split %d%s", native_kn ? "gemm_nt_dma_kernel ([K,N] operand read in place)" : use_dma ? "gemm_nt_dma_kernel" : "gemm_nt_mfma_kernel", total, splits,
                      splits > 1 ? (ln_ok ? " + splitk_reduce_ln_kernel" : " + splitk_reduce kernel") : "");
     MOON_HIP(ctx, hipGetLastError());
     if (keep_partial) {

@@ -103,6 +103,24 @@ def test_hgemm_reference_test_shapes(moon, O, ctx, M, K, N):
     assert O.rel_frobenius(ct, c) <= TOL
 
 
+# A [K, N] operand read in place (hgemm.zig:210-216) against the same product over a transposed copy: the two paths multiply
+# and add in the same order, so the results are the same bits.  Vision shapes (with and without a split of K), a partial last
+# k-tile (K = 16 * 71), ragged last tiles in m and n, one k-step, one row.
+@pytest.mark.parametrize("M,K,N", [(729, 1152, 4304), (729, 4304, 1152), (300, 1136, 1000), (130, 2064, 264), (64, 16, 8), (1, 32, 128),
+                                   (729, 1152, 1152)])
+def test_hgemm_operand_read_in_place_equals_the_transposed_copy(moon, O, ctx, monkeypatch, M, K, N):
+    a = O.fill_normal_f16((M, K), 6, 0, 1.0)
+    b = O.fill_normal_f16((K, N), 6, 1, 0.05)
+    c = moon.hgemm.matmul(a, b, ctx=ctx)
+    assert "read in place" in ctx.last_kernel()
+    monkeypatch.setenv("MOON_GEMM_KN_TRANSPOSE", "1")
+    ct = moon.hgemm.matmul(a, b, ctx=ctx)
+    assert "read in place" not in ctx.last_kernel()
+    monkeypatch.delenv("MOON_GEMM_KN_TRANSPOSE")
+    assert np.array_equal(c.view(np.uint16), ct.view(np.uint16))
+    assert O.rel_frobenius(c, O.hgemm(a, b)) <= TOL
+
+
 def test_hgemm_known_answers(moon, O, ctx):
     # A x I = A (matmul_test.zig:251-276)
     a = O.fill_normal_f16((32, 32), 2, 0, 1.0)
