@@ -262,22 +262,23 @@ def test_prefill_with_out_proj_and_fc2_in_one_launch(moon, O, ctx, monkeypatch):
 
 
 def test_prefill_with_the_rotation_in_the_qkv_product(moon, O, ctx, monkeypatch):
-    """Where the qkv projection takes the 192- / 256-row kernels its epilogue rotates q and k and writes the cache rows
-    itself; MOON_GEMM_NO_ROPE runs the projection and the rotation as two launches.  The same values, roundings and
-    rotations: hidden states, logits and the ids decoded from the cache are the same bits, for a ragged first chunk at
-    position 0 and a second chunk that starts at position 333."""
+    """Where the qkv projection takes the 192- / 256-row kernels (more 128 x 128 tiles than compute units: from 641 rows on at
+    this width) its epilogue rotates q and k and writes the cache rows itself; MOON_GEMM_NO_ROPE runs the projection and the
+    rotation as two launches.  The same values, roundings and rotations: hidden states, logits and the ids decoded from the
+    cache are the same bits, for a ragged first chunk at position 0 (700 rows: 192-row tiles, the last one partial) and a
+    second chunk that starts at position 700 (1000 rows: 256-row tiles)."""
     cfg = dict(O.TEXT_CFG, n_layers=2, vocab=2048)
     ref, dev = _text_pair(moon, O, ctx, cfg, seed=5)
-    a, b = O.fill_uniform_u32(333, 0, 52, cfg["vocab"]), O.fill_uniform_u32(200, 0, 53, cfg["vocab"])
+    a, b = O.fill_uniform_u32(700, 0, 52, cfg["vocab"]), O.fill_uniform_u32(1000, 0, 53, cfg["vocab"])
     out = []
     for fused in (True, False):
         if not fused:
             monkeypatch.setenv("MOON_GEMM_NO_ROPE", "1")
         dev.reset()
         dev.forward(a)
-        h1 = dev.hidden(333).copy()
+        h1 = dev.hidden(700).copy()
         dev.forward(b)
-        h2, lg = dev.hidden(200).copy(), dev.logits().copy()
+        h2, lg = dev.hidden(1000).copy(), dev.logits().copy()
         out.append((h1, h2, lg, dev.greedy(6).tolist()))
     monkeypatch.delenv("MOON_GEMM_NO_ROPE")
     dev.close()
