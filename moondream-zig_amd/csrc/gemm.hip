@@ -600,7 +600,8 @@ template <int MI> struct Dma2 {
 // PARTIAL: the workgroup multiplies k-tiles [kt0, kt0 + n_ktiles) of tile `wg` only and leaves the f32 sums in slab `split` of
 // p.partial (no epilogue); otherwise the whole of K, and wg is taken from the workgroup index.
 // ROPE: the epilogue of a qkv projection that writes the rotated q and the cache rows (gemm_tile_out_rope) instead of C.
-template <int EPI, int MI, bool PARTIAL = false, bool ROPE = false>
+// BKN: the second operand is [K, N], read in place as in gemm_nt_dma_kernel<EPI, true>.
+template <int EPI, int MI, bool PARTIAL = false, bool ROPE = false, bool BKN = false>
 __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p, int wg_arg = 0, int kt0 = 0, int n_ktiles_arg = 0, int split = 0) {
     static_assert(MI == 3 || MI == 4, "192- or 256-row tiles");
     static_assert(!PARTIAL || EPI == MOON_EPI_NONE, "partial sums take no epilogue");
@@ -638,10 +639,15 @@ __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p, int wg_arg 
         for (int j = 0; j < 4; j++) {
             const int r = 32 * role_wave + 8 * j + (lane >> 3);
             off_w[j] = (min(n0 + r, p.N - 1) * p.K + swz(r, lane & 7) * 8) * 2;
+            if (BKN) { // k-rows 16 * role_wave + 4 * j .. + 3 of the tile; columns past N re-read the row's last granule and are never stored
+                const int rk = 16 * role_wave + 4 * j + (lane >> 4), pg = lane & 15;
+                off_w[j] = (rk * p.N + min(n0 + (pg ^ (2 * (rk & 3))) * 8, p.N - 8)) * 2;
+            }
         }
         auto issue = [&](int kt) {
             half_t *stage = lds2 + size_t(kt % DMA2_STAGES) * STAGE2_HALFS;
             const int k_off = (kt0 + kt) * BK * 2;
+            const int kw_off = BKN ? (kt0 + kt) * BK * p.N * 2 : k_off;
 #pragma unroll
             for (int j = 0; j < A_LOADS; j++)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, (__attribute__((address_space(3))) void *)(stage + (16 * MI * role_wave + 8 * j) * BK),
@@ -649,7 +655,7 @@ __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p, int wg_arg 
 #pragma unroll
             for (int j = 0; j < 4; j++)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                    rs_w, (__attribute__((address_space(3))) void *)(stage + BM2 * BK + (32 * role_wave + 8 * j) * BK), 16, off_w[j], k_off, 0, 0);
+                    rs_w, (__attribute__((address_space(3))) void *)(stage + BM2 * BK + (32 * role_wave + 8 * j) * BK), 16, off_w[j], kw_off, 0, 0);
         };
         int issued = 0;
         // this wavefront's part of tile kt has landed once at most (A_LOADS + 4) * (issued - 1 - kt) of its copies are outstanding
@@ -703,62 +709,98 @@ __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p, int wg_arg 
             off_w[s][i] = (BM2 * BK + rn * BK + swz(rn, 2 * s + frag_g) * 8) * 2;
         }
     }
+    unsigned off_wk[2]; // BKN: see gemm_nt_dma_kernel
+#pragma unroll
+    for (int ni = 0; ni < 2; ni++) {
+        const int i = lane & 15, row = 8 * frag_g + (i >> 2);
+        const int c = wn * 8 + ni * 4 + ((lane >> 4) & 1) * 2 + ((i & 3) >> 1);
+        off_wk[ni] = (BM2 * BK + row * BN + (c ^ (2 * (row & 3))) * 8 + (i & 1) * 4) * 2;
+    }
     // (reads and waits by hand, as in the 128 x 128 kernel: MI + 2 reads per slice, one slice ahead of its 2 * MI MFMAs)
     constexpr unsigned STAGE_BYTES = STAGE2_HALFS * sizeof(half_t);
-    auto read_frags = [&](int kt, int s, half8_t (&fa)[MI], half8_t (&fw)[2]) {
+    struct Frag {
+        half8_t fa[MI], fw[2];
+        half4_t wk[2][2]; // BKN: fw[ni] arrives as two 8-byte halves
+    };
+    auto read_frags = [&](int kt, int s, Frag &f) {
         const unsigned sb = unsigned(kt % DMA2_STAGES) * STAGE_BYTES;
 #pragma unroll
-        for (int i = 0; i < MI; i++) asm volatile("ds_read_b128 %0, %1" : "=v"(fa[i]) : "v"(sb + off_a[s][i]));
+        for (int i = 0; i < MI; i++) asm volatile("ds_read_b128 %0, %1" : "=v"(f.fa[i]) : "v"(sb + off_a[s][i]));
 #pragma unroll
-        for (int i = 0; i < 2; i++) asm volatile("ds_read_b128 %0, %1" : "=v"(fw[i]) : "v"(sb + off_w[s][i]));
+        for (int i = 0; i < 2; i++) {
+            if (!BKN) asm volatile("ds_read_b128 %0, %1" : "=v"(f.fw[i]) : "v"(sb + off_w[s][i]));
+            else {
+#pragma unroll
+                for (int q = 0; q < 2; q++)
+                    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(f.wk[i][q]) : "v"(sb + off_wk[i] + unsigned(16 * s + 4 * q) * (BN * 2)));
+            }
+        }
     };
-    auto wait_older = [&](half8_t (&fa)[MI], half8_t (&fw)[2]) {
-        if constexpr (MI == 4)
-            asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[MI - 1]), "+v"(fw[0]), "+v"(fw[1])::"memory");
-        else
-            asm volatile("s_waitcnt lgkmcnt(5)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fw[0]), "+v"(fw[1])::"memory");
+    // (all but the newest group of reads have landed: MI + 2 reads a group, MI + 4 with BKN)
+    auto wait_older = [&](Frag &f) {
+        if constexpr (!BKN) {
+            if constexpr (MI == 4)
+                asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.fa[2]), "+v"(f.fa[MI - 1]), "+v"(f.fw[0]), "+v"(f.fw[1])::"memory");
+            else
+                asm volatile("s_waitcnt lgkmcnt(5)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.fa[2]), "+v"(f.fw[0]), "+v"(f.fw[1])::"memory");
+        } else {
+            if constexpr (MI == 4)
+                asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.fa[2]), "+v"(f.fa[MI - 1]), "+v"(f.wk[0][0]), "+v"(f.wk[0][1]), "+v"(f.wk[1][0]), "+v"(f.wk[1][1])::"memory");
+            else
+                asm volatile("s_waitcnt lgkmcnt(7)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.fa[2]), "+v"(f.wk[0][0]), "+v"(f.wk[0][1]), "+v"(f.wk[1][0]), "+v"(f.wk[1][1])::"memory");
+        }
     };
-    auto wait_all = [&](half8_t (&fa)[MI], half8_t (&fw)[2]) {
-        if constexpr (MI == 4)
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[MI - 1]), "+v"(fw[0]), "+v"(fw[1])::"memory");
-        else
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fw[0]), "+v"(fw[1])::"memory");
+    auto wait_all = [&](Frag &f) {
+        if constexpr (!BKN) {
+            if constexpr (MI == 4)
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.fa[2]), "+v"(f.fa[MI - 1]), "+v"(f.fw[0]), "+v"(f.fw[1])::"memory");
+            else
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.fa[2]), "+v"(f.fw[0]), "+v"(f.fw[1])::"memory");
+        } else {
+            if constexpr (MI == 4)
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.fa[2]), "+v"(f.fa[MI - 1]), "+v"(f.wk[0][0]), "+v"(f.wk[0][1]), "+v"(f.wk[1][0]), "+v"(f.wk[1][1])::"memory");
+            else
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.fa[0]), "+v"(f.fa[1]), "+v"(f.fa[2]), "+v"(f.wk[0][0]), "+v"(f.wk[0][1]), "+v"(f.wk[1][0]), "+v"(f.wk[1][1])::"memory");
+        }
     };
-    auto multiply = [&](const half8_t (&fa)[MI], const half8_t (&fw)[2]) {
+    auto multiply = [&](const Frag &f) {
+        half8_t w[2];
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++) w[ni] = BKN ? __builtin_shufflevector(f.wk[ni][0], f.wk[ni][1], 0, 1, 2, 3, 4, 5, 6, 7) : f.fw[ni];
 #pragma unroll
         for (int mi = 0; mi < MI; mi++)
 #pragma unroll
-            for (int ni = 0; ni < 2; ni++) acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[ni], fa[mi], acc[ni][mi], 0, 0, 0);
+            for (int ni = 0; ni < 2; ni++) acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w[ni], f.fa[mi], acc[ni][mi], 0, 0, 0);
     };
 
-    half8_t fa[2][MI], fw[2][2];
+    Frag fr[2];
     lds_barrier(); // tile 0 is visible
-    read_frags(0, 0, fa[0], fw[0]);
+    read_frags(0, 0, fr[0]);
     auto first_three = [&](int kt) {
-        read_frags(kt, 1, fa[1], fw[1]);
-        wait_older(fa[0], fw[0]);
-        multiply(fa[0], fw[0]);
+        read_frags(kt, 1, fr[1]);
+        wait_older(fr[0]);
+        multiply(fr[0]);
         __builtin_amdgcn_sched_barrier(0);
-        read_frags(kt, 2, fa[0], fw[0]);
-        wait_older(fa[1], fw[1]);
-        multiply(fa[1], fw[1]);
+        read_frags(kt, 2, fr[0]);
+        wait_older(fr[1]);
+        multiply(fr[1]);
         __builtin_amdgcn_sched_barrier(0);
-        read_frags(kt, 3, fa[1], fw[1]);
-        wait_older(fa[0], fw[0]);
-        multiply(fa[0], fw[0]);
+        read_frags(kt, 3, fr[1]);
+        wait_older(fr[0]);
+        multiply(fr[0]);
         __builtin_amdgcn_sched_barrier(0);
     };
     for (int kt = 0; kt + 1 < n_ktiles; kt++) { // (every k-tile is a full one)
         first_three(kt);
-        wait_all(fa[1], fw[1]);
+        wait_all(fr[1]);
         __builtin_amdgcn_s_barrier();
-        read_frags(kt + 1, 0, fa[0], fw[0]);
-        multiply(fa[1], fw[1]);
+        read_frags(kt + 1, 0, fr[0]);
+        multiply(fr[1]);
         __builtin_amdgcn_sched_barrier(0);
     }
     first_three(n_ktiles - 1);
-    wait_all(fa[1], fw[1]);
-    multiply(fa[1], fw[1]);
+    wait_all(fr[1]);
+    multiply(fr[1]);
     if constexpr (SHARED_EPILOGUE) {
         // With GELU the epilogue is VALU work and the loaders have nothing left to do: the multipliers park the whole tile in
         // LDS as f16 ([m][n], pitch 136 halfs, from the start of the staging area, which is free once every multiplier has
@@ -833,13 +875,13 @@ __device__ __forceinline__ void gemm_nt_dma2_body(const GemmArgs &p, int wg_arg 
 }
 
 // (the two tile heights as kernels of their own with one template parameter, like the other kernels of this file)
-template <int EPI>
+template <int EPI, bool BKN = false>
 __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma256_kernel(GemmArgs p) {
-    gemm_nt_dma2_body<EPI, 4>(p);
+    gemm_nt_dma2_body<EPI, 4, false, false, BKN>(p);
 }
-template <int EPI>
+template <int EPI, bool BKN = false>
 __global__ __launch_bounds__(DMA_THREADS) void gemm_nt_dma192_kernel(GemmArgs p) {
-    gemm_nt_dma2_body<EPI, 3>(p);
+    gemm_nt_dma2_body<EPI, 3, false, false, BKN>(p);
 }
 
 // A decoder block's qkv projection with the rotation and the cache update in its epilogue (one kernel per tile height)
@@ -1049,18 +1091,6 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
         return MOON_OK;
     }
     const half_t *Bt = B;
-    // A [K, N] operand is read as it lies by the 128 x 128 wavefront-specialised kernel where the shape takes that kernel
-    // (at most one tile per compute unit); other shapes get a transposed copy first.  MOON_GEMM_KN_TRANSPOSE: always the copy.
-    const bool native_kn = b_layout == MOON_B_KN && N % 8 == 0 && K % 16 == 0 && size_t(M) * K * 2 < (size_t(1) << 31) - 4096 &&
-                           size_t(N) * K * 2 < (size_t(1) << 31) - 4096 && !ctx->gemm_kernel[0] && !getenv("MOON_GEMM_KN_TRANSPOSE") &&
-                           size_t((M + BM - 1) / BM) * ((N + BN - 1) / BN) <= size_t(ctx->cu_count > 0 ? ctx->cu_count : 256);
-    if (b_layout == MOON_B_KN && !native_kn) {
-        MOON_TRY(moon_grow(ctx, ctx->work[2], size_t(N) * K * sizeof(half_t)));
-        hipLaunchKernelGGL(transpose_kernel, dim3((N + 63) / 64, (K + 63) / 64), dim3(256), 0, ctx->stream, B,
-                           (half_t *)ctx->work[2].ptr, K, N);
-        MOON_HIP(ctx, hipGetLastError());
-        Bt = (const half_t *)ctx->work[2].ptr;
-    }
     GemmArgs p;
     p.A = A;
     p.Bt = Bt;
@@ -1098,6 +1128,18 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
     if (wide_ok && force && !strcmp(force, "w114")) wide = 114;
     if (wide_ok && force && !strcmp(force, "w212")) wide = 212;
     if (wide_ok && force && !strcmp(force, "w221")) wide = 221;
+    // A [K, N] operand is read as it lies by the wavefront-specialised kernels (the 128 x 128 one up to one tile per compute
+    // unit, the 192- / 256-row ones beyond); the other kernels get a transposed copy first.  MOON_GEMM_KN_TRANSPOSE: always the copy.
+    const bool native_kn = b_layout == MOON_B_KN && N % 8 == 0 && K % 16 == 0 && buffers_ok && !force && !wide && !getenv("MOON_GEMM_KN_TRANSPOSE") &&
+                           (tiles <= cus || (K % BK == 0 && p.lds_epilogue));
+    if (b_layout == MOON_B_KN && !native_kn) {
+        MOON_TRY(moon_grow(ctx, ctx->work[2], size_t(N) * K * sizeof(half_t)));
+        hipLaunchKernelGGL(transpose_kernel, dim3((N + 63) / 64, (K + 63) / 64), dim3(256), 0, ctx->stream, B,
+                           (half_t *)ctx->work[2].ptr, K, N);
+        MOON_HIP(ctx, hipGetLastError());
+        Bt = (const half_t *)ctx->work[2].ptr;
+        p.Bt = Bt;
+    }
     if (wide) {
         const int tm = wide == 114 ? 128 : 256, tn = wide == 221 ? 256 : 128;
         p.tiles_m = (M + tm - 1) / tm;
@@ -1176,17 +1218,22 @@ int run_gemm(moon_ctx *ctx, const half_t *A, const half_t *B, const half_t *bias
         const int total = p.tiles_m * p.tiles_n;
         const size_t lds_bytes = use192 ? Dma2<3>::LDS_BYTES : Dma2<4>::LDS_BYTES;
         // the opt-in to this much dynamic LDS is per device and per kernel (here: per epilogue instantiation); setting it twice is harmless
-        static std::atomic<bool> attr_set[2][64];
+        static std::atomic<bool> attr_set[4][64];
         const int dev = ctx->device >= 0 && ctx->device < 64 ? ctx->device : -1;
-        if (dev < 0 || !attr_set[use192 ? 1 : 0][dev].load()) {
-            const void *kern = use192 ? reinterpret_cast<const void *>(gemm_nt_dma192_kernel<EPI>) : reinterpret_cast<const void *>(gemm_nt_dma256_kernel<EPI>);
+        const int which = (use192 ? 1 : 0) + (native_kn ? 2 : 0);
+        if (dev < 0 || !attr_set[which][dev].load()) {
+            const void *kern = native_kn ? (use192 ? reinterpret_cast<const void *>(gemm_nt_dma192_kernel<EPI, true>) : reinterpret_cast<const void *>(gemm_nt_dma256_kernel<EPI, true>))
+                                         : (use192 ? reinterpret_cast<const void *>(gemm_nt_dma192_kernel<EPI>) : reinterpret_cast<const void *>(gemm_nt_dma256_kernel<EPI>));
             MOON_HIP(ctx, hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-            if (dev >= 0) attr_set[use192 ? 1 : 0][dev].store(true);
+            if (dev >= 0) attr_set[which][dev].store(true);
         }
         const dim3 grid2(((total + 7) / 8) * 8);
-        if (use192) hipLaunchKernelGGL(gemm_nt_dma192_kernel<EPI>, grid2, dim3(DMA_THREADS), lds_bytes, ctx->stream, p);
+        if (native_kn) {
+            if (use192) hipLaunchKernelGGL((gemm_nt_dma192_kernel<EPI, true>), grid2, dim3(DMA_THREADS), lds_bytes, ctx->stream, p);
+            else hipLaunchKernelGGL((gemm_nt_dma256_kernel<EPI, true>), grid2, dim3(DMA_THREADS), lds_bytes, ctx->stream, p);
+        } else if (use192) hipLaunchKernelGGL(gemm_nt_dma192_kernel<EPI>, grid2, dim3(DMA_THREADS), lds_bytes, ctx->stream, p);
         else hipLaunchKernelGGL(gemm_nt_dma256_kernel<EPI>, grid2, dim3(DMA_THREADS), lds_bytes, ctx->stream, p);
-        MOON_NOTE_KERNEL(ctx, "%s %d workgroups", use192 ? "gemm_nt_dma192_kernel" : "gemm_nt_dma256_kernel", total);
+        MOON_NOTE_KERNEL(ctx, "%s%s %d workgroups", use192 ? "gemm_nt_dma192_kernel" : "gemm_nt_dma256_kernel", native_kn ? " ([K,N] operand read in place)" : "", total);
         MOON_HIP(ctx, hipGetLastError());
         return MOON_OK;
     }

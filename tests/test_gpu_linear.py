@@ -105,9 +105,11 @@ def test_hgemm_reference_test_shapes(moon, O, ctx, M, K, N):
 
 # A [K, N] operand read in place (hgemm.zig:210-216) against the same product over a transposed copy: the two paths multiply
 # and add in the same order, so the results are the same bits.  Vision shapes (with and without a split of K), a partial last
-# k-tile (K = 16 * 71), ragged last tiles in m and n, one k-step, one row.
+# k-tile (K = 16 * 71), ragged last tiles in m and n, one k-step, one row, and shapes that take the larger tiles.
 @pytest.mark.parametrize("M,K,N", [(729, 1152, 4304), (729, 4304, 1152), (300, 1136, 1000), (130, 2064, 264), (64, 16, 8), (1, 32, 128),
-                                   (729, 1152, 1152)])
+                                   (729, 1152, 1152),
+                                   # more tiles than compute units: the 256- and the 192-row kernels, the latter also with a ragged last column tile
+                                   (1458, 1152, 4304), (768, 2048, 8192), (700, 128, 8000)])
 def test_hgemm_operand_read_in_place_equals_the_transposed_copy(moon, O, ctx, monkeypatch, M, K, N):
     a = O.fill_normal_f16((M, K), 6, 0, 1.0)
     b = O.fill_normal_f16((K, N), 6, 1, 0.05)
