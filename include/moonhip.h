@@ -428,7 +428,6 @@ int moon_bin_vision_io_weights(const moon_bin *bin, const moon_vision_config *cf
  *   MOON_LAYER_QKV_WGS=n           decode mode 0: workgroups that take qkv rows (default: the attention and output workgroups)
  *   MOON_LAYER_FC1_OUT_ROWS=n      decode mode 0: fc1 rows per output wavefront (default: about a third of an fc1-only wavefront's
  *                                  share, at least one; 0 is allowed)
- *   MOON_LAYER_FC1_GROUP=1|2       decode mode 0: fc1 rows a wavefront requests together (default 1)
  *   MOON_GEMM_KERNEL=regs|dma|dma256|w114|w212|w221  forces one of the MFMA product kernels where the shape allows it (default: by shape)
  *   MOON_GEMM_EPILOGUE=direct      the product kernels store their tile without the pass through LDS (default: through LDS)
  *   MOON_SAMPLE_SEPARATE=1         sampled loops with top_k <= 3: the LM-head launch leaves every token to sample_kernel instead of

@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void decode_attn_partial_kernel(const half_t *
                                                                    int pos_arg, const uint32_t *__restrict__ pos_dev) {
     const int pos = pos_dev ? (int)*pos_dev : pos_arg;
     const int h = blockIdx.x / DEC_SPLITS, split = blockIdx.x % DEC_SPLITS;
-    DecodeAttnPrefetch pf;
+    DecodeAttnPrefetch<> pf;
     decode_attn_prefetch<D>(pf, ck, cv, max_seq, pos, FUSED, h, split);
     decode_attn_task<D, FUSED>(qkv, ck, cv, table, partial, H, rot_dim, max_seq, pos, h, split, pf);
 }

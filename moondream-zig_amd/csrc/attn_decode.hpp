@@ -24,7 +24,7 @@ __device__ __forceinline__ void decode_attn_range(int pos_real, bool fused, int 
         j1 = min(pos_real, j0 + per);
     }
 }
-constexpr int DEC_PREFETCH = 4;                 // keys per lane group whose K and V rows are loaded up front
+constexpr int DEC_PREFETCH = 4;                 // keys per lane group whose K and V rows are loaded up front (the default of the PF parameters below)
 
 // Merge the DEC_SPLITS partials of one head in a fixed order; returns output element d of that head.
 template <int D, bool COH = false>
@@ -52,13 +52,16 @@ __device__ __forceinline__ half_t decode_attn_merge(const float *__restrict__ p 
     return (half_t)f32_round(o * (1.0f / l)); // attention.zig:612-615 multiplies by the reciprocal of the sum
 }
 
-// K and V rows of the first DEC_PREFETCH keys of every lane group of a (head, split) task.  They depend only on the
-// position, not on the new token, so a caller may request them long before it runs the task.
+// K and V rows of the first PF keys of every lane group of a (head, split) task (32 keys of the split per step: 8 lane groups in
+// each of 4 wavefronts).  They depend only on the position, not on the new token, so a caller may request them long before it
+// runs the task.  Keys past 32 * PF of a split are loaded inside the task, one dependent round trip per 32: a caller that
+// knows the position picks PF to cover the split (results do not depend on PF).
+template <int PF = DEC_PREFETCH>
 struct DecodeAttnPrefetch {
-    uint4 k[DEC_PREFETCH], v[DEC_PREFETCH];
+    uint4 k[PF], v[PF];
 };
-template <int D>
-__device__ __forceinline__ void decode_attn_prefetch(DecodeAttnPrefetch &pf, const half_t *__restrict__ ck, const half_t *__restrict__ cv,
+template <int D, int PF = DEC_PREFETCH>
+__device__ __forceinline__ void decode_attn_prefetch(DecodeAttnPrefetch<PF> &pf, const half_t *__restrict__ ck, const half_t *__restrict__ cv,
                                                      int max_seq, int pos_real, bool fused, int h, int split) {
     const int pos = fused ? pos_real : -1;
     int j0, j1;
@@ -69,7 +72,7 @@ __device__ __forceinline__ void decode_attn_prefetch(DecodeAttnPrefetch &pf, con
     const half_t *vbase = cv + size_t(h) * max_seq * D;
     const int jfirst = j0 + wave * 8 + g;
 #pragma unroll
-    for (int i = 0; i < DEC_PREFETCH; i++) {
+    for (int i = 0; i < PF; i++) {
         const int j = jfirst + 32 * i;
         pf.k[i] = make_uint4(0, 0, 0, 0);
         pf.v[i] = make_uint4(0, 0, 0, 0);
@@ -90,11 +93,11 @@ __device__ __forceinline__ void decode_attn_prefetch(DecodeAttnPrefetch &pf, con
 //      merged_out[h*D ..] and then counts the head in at done_count.
 // pf holds the rows requested by decode_attn_prefetch for the same (h, split, pos).  Workgroup synchronisation is LDS-only.
 // Every thread of the workgroup must call it.
-template <int D, bool FUSED, bool COH = false>
+template <int D, bool FUSED, bool COH = false, int PF = DEC_PREFETCH>
 __device__ __forceinline__ void decode_attn_task(const half_t *__restrict__ qkv, half_t *__restrict__ ck,
                                                  half_t *__restrict__ cv, const float *__restrict__ table,
                                                  float *__restrict__ partial, int H, int rot_dim, int max_seq, int pos_real,
-                                                 int h, int split, const DecodeAttnPrefetch &pf, uint32_t *head_count = nullptr,
+                                                 int h, int split, const DecodeAttnPrefetch<PF> &pf, uint32_t *head_count = nullptr,
                                                  uint32_t count_target = 0, half_t *merged_out = nullptr, uint32_t *done_count = nullptr) {
     static_assert(D == 64, "one 16-byte granule per lane, 8 lanes per key");
     __shared__ float sq[D];
@@ -167,11 +170,11 @@ __device__ __forceinline__ void decode_attn_task(const half_t *__restrict__ qkv,
         if (e == 0) sscore[j - j0] = s * scale;
     };
 #pragma unroll
-    for (int i = 0; i < DEC_PREFETCH; i++) {
+    for (int i = 0; i < PF; i++) {
         const int j = jfirst + 32 * i;
         if (j < j1) score(j, j == pos ? *reinterpret_cast<const uint4 *>(&sk_new[8 * e]) : pf.k[i]);
     }
-    for (int j = jfirst + 32 * DEC_PREFETCH; j < j1; j += 32)
+    for (int j = jfirst + 32 * PF; j < j1; j += 32)
         score(j, j == pos ? *reinterpret_cast<const uint4 *>(&sk_new[8 * e]) : *reinterpret_cast<const uint4 *>(kbase + size_t(j) * D + 8 * e));
     lds_barrier();
 
@@ -205,11 +208,11 @@ __device__ __forceinline__ void decode_attn_task(const half_t *__restrict__ qkv,
         for (int i = 0; i < 8; i++) acc[i] = fmaf(p, (float)vh[i], acc[i]);
     };
 #pragma unroll
-    for (int i = 0; i < DEC_PREFETCH; i++) {
+    for (int i = 0; i < PF; i++) {
         const int j = jfirst + 32 * i;
         if (j < j1) accumulate(j, j == pos ? *reinterpret_cast<const uint4 *>(&sv_new[8 * e]) : pf.v[i]);
     }
-    for (int j = jfirst + 32 * DEC_PREFETCH; j < j1; j += 32)
+    for (int j = jfirst + 32 * PF; j < j1; j += 32)
         accumulate(j, j == pos ? *reinterpret_cast<const uint4 *>(&sv_new[8 * e]) : *reinterpret_cast<const uint4 *>(vbase + size_t(j) * D + 8 * e));
 #pragma unroll
     for (int i = 0; i < 8; i++) {

@@ -547,7 +547,7 @@ __global__ __launch_bounds__(256) void decode_front_kernel(FrontArgs a) {
 
     const int pos = a.pos_dev ? (int)*a.pos_dev : a.pos;
     const int h = blockIdx.x / DEC_SPLITS, split = blockIdx.x % DEC_SPLITS;
-    DecodeAttnPrefetch pf;
+    DecodeAttnPrefetch<> pf;
     decode_attn_prefetch<64>(pf, a.ck, a.cv, a.max_seq, pos, true, h, split); // independent of the new token: in flight during the wait
     if (tid == 0) {
         // the counter alone is polled; the clock and the error word are looked at once in 64 polls
@@ -674,8 +674,10 @@ __device__ __forceinline__ float dot_row_lds(const u32x4 (&w)[CH], const half_t 
 }
 
 // FC1_GROUP: fc1 rows a wavefront requests together.  The fewer bytes a compute unit has queued, the sooner the small
-// dependent accesses of the attention chain issued from it are served.
-template <int CH_D, int CH_F, int FC1_GROUP>
+// dependent accesses of the attention chain issued from it are served (two measured 3 % slower than one).
+// PF: 32-key steps of an attention task whose K and V rows are requested before the wait for q (decode_attn_prefetch); the
+// host picks the instantiation that covers a split at the launch's position.
+template <int CH_D, int CH_F, int FC1_GROUP, int PF>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void decode_layer_kernel(LayerArgs a) {
     extern __shared__ __attribute__((aligned(16))) half_t smem[]; // [d] LayerNorm output, later attn; then [ffn] fc1
     __shared__ float s_red[16];
@@ -743,8 +745,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         const int h = b / DEC_SPLITS, split = b % DEC_SPLITS;
         // K and V rows do not depend on the new token: wavefronts 1-3 request theirs before the wait.  Wavefront 0 polls,
         // and a poll returns in order behind whatever the wavefront has in flight, so it requests its rows afterwards.
-        DecodeAttnPrefetch pf;
-        if (wave != 0) decode_attn_prefetch<64>(pf, a.ck, a.cv, a.max_seq, pos, true, h, split);
+        DecodeAttnPrefetch<PF> pf;
+        if (wave != 0) decode_attn_prefetch<64, PF>(pf, a.ck, a.cv, a.max_seq, pos, true, h, split);
         // The cached keys need q only; k and v of the new token are one more key, which the last split holds alone
         // (decode_attn_range).  So that split waits for all of the head's rows, the others for its q rows.
         if (split == DEC_SPLITS - 1) {
@@ -752,9 +754,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         } else {
             if (!wait_reached(a.sync + (LAYER_SYNC_QKV + a.H + h) * LAYER_LINE, a.generation * 64u, a.error, &s_flag)) return;
         }
-        if (wave == 0) decode_attn_prefetch<64>(pf, a.ck, a.cv, a.max_seq, pos, true, h, split);
+        if (wave == 0) decode_attn_prefetch<64, PF>(pf, a.ck, a.cv, a.max_seq, pos, true, h, split);
         stamp(2); // what this split needs of the head's q, k, v is complete
-        decode_attn_task<64, true, true>(p.y1, a.ck, a.cv, a.table, a.partial, a.H, a.rot_dim, a.max_seq, pos, h, split, pf, a.head_count,
+        decode_attn_task<64, true, true, PF>(p.y1, a.ck, a.cv, a.table, a.partial, a.H, a.rot_dim, a.max_seq, pos, h, split, pf, a.head_count,
                                          a.head_target, a.attn_out, a.sync + LAYER_SYNC_HEADS_DONE * LAYER_LINE);
         stamp(3); // task (and possibly the head's merge) done
         return;
@@ -933,7 +935,7 @@ __global__ __launch_bounds__(256) void decode_attn_merged_kernel(const half_t *_
                                                                   int max_seq, int pos_arg, const uint32_t *__restrict__ pos_dev) {
     const int pos = pos_dev ? (int)*pos_dev : pos_arg;
     const int h = blockIdx.x / DEC_SPLITS, split = blockIdx.x % DEC_SPLITS;
-    DecodeAttnPrefetch pf;
+    DecodeAttnPrefetch<> pf;
     decode_attn_prefetch<D>(pf, ck, cv, max_seq, pos, true, h, split);
     // device-coherent partials and a per-head counter: whichever split finishes a head last merges it
     decode_attn_task<D, true, true>(qkv, ck, cv, table, partial, H, rot_dim, max_seq, pos, h, split, pf, head_count, count_target, out);
@@ -1015,7 +1017,9 @@ bool decode_layer_supported(moon_ctx *ctx, size_t d, size_t ffn, size_t H, size_
     const int waiting = (int)(H * DEC_SPLITS + (d + 3) / 4); // attention and output workgroups
     if (waiting >= grid || 3 * d > size_t(16) * grid) return false;
     int per_cu = 0;
-    const void *kernels[2] = {reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 1>), reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 2>)};
+    const void *kernels[5] = {reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 1, 4>), reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 1, 5>),
+                              reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 1, 6>), reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 1, 8>),
+                              reinterpret_cast<const void *>(decode_layer_kernel<4, 16, 1, 10>)};
     for (const void *k : kernels) {
         if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)((d + ffn) * sizeof(half_t))) != hipSuccess) return false;
         int n = 0;
@@ -1081,13 +1085,17 @@ int launch_decode_layer(moon_ctx *ctx, const half_t *x, const uint32_t *token, c
     a.ffn = (int)ffn;
     a.pos_dev = pos_dev;
     const unsigned grid = (unsigned)(LN_GEMV_GROUPS_PER_CU * (ctx->cu_count > 0 ? ctx->cu_count : 256));
-    static int group = 0;
-    if (!group) {
-        const char *e = getenv("MOON_LAYER_FC1_GROUP");
-        group = e && atoi(e) == 2 ? 2 : 1;
-    }
-    if (group == 2) hipLaunchKernelGGL((decode_layer_kernel<4, 16, 2>), dim3(grid), dim3(256), (d + ffn) * sizeof(half_t), ctx->stream, a);
-    else hipLaunchKernelGGL((decode_layer_kernel<4, 16, 1>), dim3(grid), dim3(256), (d + ffn) * sizeof(half_t), ctx->stream, a);
+    // The instantiation whose attention tasks request all their K and V rows before the wait for q: the pos cached keys go to
+    // DEC_SPLITS - 1 splits, 32 keys per prefetch step (a step too few costs a dependent round trip per 32 keys inside the
+    // attention chain: 0.628 instead of 0.598 ms per token at 900-1030 cached keys; steps too many cost 1-2 % at short
+    // contexts).  pos is the host's count; a loop that has stopped at an end-of-sequence token only over-provides.
+    const size_t per_split = (pos + DEC_SPLITS - 2) / (DEC_SPLITS - 1), steps = (per_split + 31) / 32;
+    const size_t lds = (d + ffn) * sizeof(half_t);
+    if (steps <= 4) hipLaunchKernelGGL((decode_layer_kernel<4, 16, 1, 4>), dim3(grid), dim3(256), lds, ctx->stream, a);
+    else if (steps <= 5) hipLaunchKernelGGL((decode_layer_kernel<4, 16, 1, 5>), dim3(grid), dim3(256), lds, ctx->stream, a);
+    else if (steps <= 6) hipLaunchKernelGGL((decode_layer_kernel<4, 16, 1, 6>), dim3(grid), dim3(256), lds, ctx->stream, a);
+    else if (steps <= 8) hipLaunchKernelGGL((decode_layer_kernel<4, 16, 1, 8>), dim3(grid), dim3(256), lds, ctx->stream, a);
+    else hipLaunchKernelGGL((decode_layer_kernel<4, 16, 1, 10>), dim3(grid), dim3(256), lds, ctx->stream, a);
     MOON_HIP(ctx, hipGetLastError());
     return MOON_OK;
 }
