@@ -164,9 +164,11 @@ __device__ __forceinline__ void decode_attn_task(const half_t *__restrict__ qkv,
         float s = 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; i++) s = fmaf(qf[i], (float)kh[i], s);
-        s += __shfl_xor(s, 1, 64);
-        s += __shfl_xor(s, 2, 64);
-        s += __shfl_xor(s, 4, 64);
+        // the 8 lanes' sum on the DPP path (swap within pairs, swap pairs, mirror the 8): the same additions as an xor butterfly
+        // over 1, 2, 4 (each level adds the same two values, in either order), without three trips through the LDS crossbar
+        s += dpp_move<DPP_QUAD_XOR1>(s);
+        s += dpp_move<DPP_QUAD_XOR2>(s);
+        s += dpp_move<DPP_ROW_HALF_MIRROR>(s);
         if (e == 0) sscore[j - j0] = s * scale;
     };
 #pragma unroll
