@@ -488,7 +488,7 @@ struct FrontArgs {
 constexpr long long FRONT_TIMEOUT_TICKS = 100000000LL; // 1 s of the 100 MHz wall clock
 constexpr int FRONT_COUNTER_STRIDE = 32;               // uint32 slots per 128-byte line: one line per head
 
-template <int CH>
+template <int CH, int PF>
 __global__ __launch_bounds__(256) void decode_front_kernel(FrontArgs a) {
     extern __shared__ __attribute__((aligned(16))) half_t s_ln[]; // [d]
     __shared__ float s_red[16];
@@ -547,8 +547,8 @@ __global__ __launch_bounds__(256) void decode_front_kernel(FrontArgs a) {
 
     const int pos = a.pos_dev ? (int)*a.pos_dev : a.pos;
     const int h = blockIdx.x / DEC_SPLITS, split = blockIdx.x % DEC_SPLITS;
-    DecodeAttnPrefetch<> pf;
-    decode_attn_prefetch<64>(pf, a.ck, a.cv, a.max_seq, pos, true, h, split); // independent of the new token: in flight during the wait
+    DecodeAttnPrefetch<PF> pf;
+    decode_attn_prefetch<64, PF>(pf, a.ck, a.cv, a.max_seq, pos, true, h, split); // independent of the new token: in flight during the wait
     if (tid == 0) {
         // the counter alone is polled; the clock and the error word are looked at once in 64 polls
         const long long t0 = wall_clock64();
@@ -572,7 +572,7 @@ __global__ __launch_bounds__(256) void decode_front_kernel(FrontArgs a) {
     lds_barrier();
     if (!s_ok) return;
     // q, k and v of this head are complete
-    decode_attn_task<64, true, true>(p.y1, a.ck, a.cv, a.table, a.partial, a.H, a.rot_dim, a.max_seq, pos, h, split, pf, a.head_count,
+    decode_attn_task<64, true, true, PF>(p.y1, a.ck, a.cv, a.table, a.partial, a.H, a.rot_dim, a.max_seq, pos, h, split, pf, a.head_count,
                                      a.head_target, a.attn_out);
 }
 
@@ -927,7 +927,7 @@ __global__ __launch_bounds__(256) void decode_out_fc2_kernel(OutFc2Args p) {
     }
 }
 
-template <int D>
+template <int D, int PF>
 __global__ __launch_bounds__(256) void decode_attn_merged_kernel(const half_t *__restrict__ qkv, half_t *__restrict__ ck,
                                                                   half_t *__restrict__ cv, const float *__restrict__ table,
                                                                   float *__restrict__ partial, half_t *__restrict__ out,
@@ -935,10 +935,10 @@ __global__ __launch_bounds__(256) void decode_attn_merged_kernel(const half_t *_
                                                                   int max_seq, int pos_arg, const uint32_t *__restrict__ pos_dev) {
     const int pos = pos_dev ? (int)*pos_dev : pos_arg;
     const int h = blockIdx.x / DEC_SPLITS, split = blockIdx.x % DEC_SPLITS;
-    DecodeAttnPrefetch<> pf;
-    decode_attn_prefetch<D>(pf, ck, cv, max_seq, pos, true, h, split);
+    DecodeAttnPrefetch<PF> pf;
+    decode_attn_prefetch<D, PF>(pf, ck, cv, max_seq, pos, true, h, split);
     // device-coherent partials and a per-head counter: whichever split finishes a head last merges it
-    decode_attn_task<D, true, true>(qkv, ck, cv, table, partial, H, rot_dim, max_seq, pos, h, split, pf, head_count, count_target, out);
+    decode_attn_task<D, true, true, PF>(qkv, ck, cv, table, partial, H, rot_dim, max_seq, pos, h, split, pf, head_count, count_target, out);
 }
 
 // sampling.argmax (sampling.zig:257-273) + bookkeeping of the greedy loop: state[2] = token, out_ids[state[1]++] = token.
@@ -1108,7 +1108,7 @@ bool decode_front_supported(moon_ctx *ctx, size_t d, size_t H, size_t D) {
     const int grid = LN_GEMV_GROUPS_PER_CU * cus;
     if ((int)(H * DEC_SPLITS) >= grid || 3 * d > size_t(16) * grid) return false; // every wavefront's qkv rows fit its first group
     int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(decode_front_kernel<4>), 256, d * sizeof(half_t)) !=
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(decode_front_kernel<4, 10>), 256, d * sizeof(half_t)) !=
         hipSuccess)
         return false;
     return per_cu * cus >= 2 * (int)(H * DEC_SPLITS);
@@ -1140,7 +1140,8 @@ int launch_decode_front(moon_ctx *ctx, const half_t *x, const uint32_t *token, c
     a.pos = (int)pos;
     a.pos_dev = pos_dev;
     const unsigned grid = (unsigned)(LN_GEMV_GROUPS_PER_CU * (ctx->cu_count > 0 ? ctx->cu_count : 256));
-    hipLaunchKernelGGL(decode_front_kernel<4>, dim3(grid), dim3(256), d * sizeof(half_t), ctx->stream, a);
+    if ((pos + DEC_SPLITS - 2) / (DEC_SPLITS - 1) <= 128) hipLaunchKernelGGL((decode_front_kernel<4, 4>), dim3(grid), dim3(256), d * sizeof(half_t), ctx->stream, a);
+    else hipLaunchKernelGGL((decode_front_kernel<4, 10>), dim3(grid), dim3(256), d * sizeof(half_t), ctx->stream, a);
     MOON_HIP(ctx, hipGetLastError());
     return MOON_OK;
 }
@@ -1249,8 +1250,13 @@ int launch_decode_attention_merged(moon_ctx *ctx, const half_t *qkv, half_t *cac
                                    size_t max_seq, size_t pos, const uint32_t *pos_dev) {
     if (D != 64) return moon_fail(ctx, MOON_EINVAL_DIM, "decode attention: head_dim %zu unsupported (64 only)", D);
     if (max_seq > 2048 || pos >= max_seq) return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "decode attention: pos %zu >= max_seq %zu (limit 2048)", pos, max_seq);
-    hipLaunchKernelGGL(decode_attn_merged_kernel<64>, dim3((unsigned)(H * DEC_SPLITS)), dim3(256), 0, ctx->stream, qkv, cache_k, cache_v, table,
-                       partial, out, head_count, count_target, (int)H, (int)rot_dim, (int)max_seq, (int)pos, pos_dev);
+    // (two prefetch depths: up to 4 steps of 32 keys per split, which is 896 cached keys, and everything beyond; see launch_decode_layer)
+    if ((pos + DEC_SPLITS - 2) / (DEC_SPLITS - 1) <= 128)
+        hipLaunchKernelGGL((decode_attn_merged_kernel<64, 4>), dim3((unsigned)(H * DEC_SPLITS)), dim3(256), 0, ctx->stream, qkv, cache_k, cache_v, table,
+                           partial, out, head_count, count_target, (int)H, (int)rot_dim, (int)max_seq, (int)pos, pos_dev);
+    else
+        hipLaunchKernelGGL((decode_attn_merged_kernel<64, 10>), dim3((unsigned)(H * DEC_SPLITS)), dim3(256), 0, ctx->stream, qkv, cache_k, cache_v, table,
+                           partial, out, head_count, count_target, (int)H, (int)rot_dim, (int)max_seq, (int)pos, pos_dev);
     MOON_HIP(ctx, hipGetLastError());
     MOON_NOTE_KERNEL(ctx, "decode_attn_merged_kernel<64> %d workgroups", (int)(H * DEC_SPLITS));
     return MOON_OK;

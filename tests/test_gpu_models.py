@@ -291,6 +291,31 @@ def test_prefill_with_the_rotation_in_the_qkv_product(moon, O, ctx, monkeypatch)
     assert O.rel_frobenius(out[0][1], h_ref) <= TOL
 
 
+@pytest.mark.parametrize("prompt", [880, 1000, 1200, 1500, 1900])
+def test_decode_modes_agree_at_long_contexts(moon, O, ctx, prompt):
+    """The one-launch-per-layer kernel is instantiated for several prefetch depths of its attention tasks and the host picks
+    one by the position (4, 5, 6, 8 and 10 steps of 32 keys per split at these prompt lengths; the other modes have two
+    depths).  The depth only changes when a key is requested: the modes agree bit for bit at every context length, and at
+    the shortest and the longest of them the decoded ids and logits match the oracle's."""
+    cfg = dict(O.TEXT_CFG, n_layers=2, vocab=2048)
+    ref, dev = _text_pair(moon, O, ctx, cfg, seed=7)
+    ids = O.fill_uniform_u32(prompt, 0, 55, cfg["vocab"])
+    (t1, l1, p1), *others = _all_modes(dev, ids, 10)
+    assert p1 == prompt + 10
+    for t, l, p in others:
+        assert t == t1 and p == p1
+        assert np.array_equal(l.view(np.uint16), l1.view(np.uint16))
+    dev.close()
+    if prompt in (880, 1900):
+        want, margins, ref_logits = ref.greedy(ids, 11)  # (the session's logits after 10 tokens are those that pick the 11th)
+        for step, (got, exp, margin) in enumerate(zip(t1, want, margins)):
+            if margin < 2e-2:  # (a near-tie in the oracle's own logits: either token is within the products' tolerance)
+                break
+            assert got == exp, f"step {step}: {got} != {exp} (oracle top-2 margin {margin:.4f})"
+        else:
+            assert O.rel_frobenius(l1.reshape(1, -1), ref_logits[-1].reshape(1, -1)) <= TOL
+
+
 def test_sessions_built_from_a_moondream_bin_file(moon, O, ctx, tmp_path):
     """Weights written in the reference's file layout, mapped by the library's reader and uploaded from the mapping: the
     decoder and the vision encoder give the same bits as when built from in-memory arrays, and match the oracle."""
