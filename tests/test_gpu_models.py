@@ -261,6 +261,21 @@ def test_prefill_with_out_proj_and_fc2_in_one_launch(moon, O, ctx, monkeypatch):
     assert max(errs) <= TOL
 
 
+@pytest.mark.parametrize("dim,hidden,heads,rows", [(512, 2048, 8, 300), (1024, 4096, 16, 700), (256, 1024, 4, 200)])
+def test_prefill_of_other_widths_through_the_joint_launch(moon, O, ctx, dim, hidden, heads, rows):
+    """The joint out_proj + fc2 launch at other model widths (its splits of K and its tile counts follow the shape), on
+    prompts long enough to take it: hidden states, logits and the ids decoded afterwards against the oracle."""
+    cfg = dict(vocab=1500, dim=dim, hidden_dim=hidden, n_layers=3, n_heads=heads, head_dim=64, rot_dim=32, theta=10000.0, max_seq=1024)
+    ref, dev = _text_pair(moon, O, ctx, cfg, seed=8)
+    ids = O.fill_uniform_u32(rows, 0, 56, cfg["vocab"])
+    cache = ref.new_cache()
+    h_ref = ref.text_decoder(ref.text_encoder(ids), cache)
+    dev.forward(ids)
+    assert O.rel_frobenius(dev.hidden(rows), h_ref) <= TOL
+    assert O.rel_frobenius(dev.logits().reshape(1, -1), ref.lm_head(h_ref).reshape(1, -1)) <= TOL
+    dev.close()
+
+
 def test_prefill_with_the_rotation_in_the_qkv_product(moon, O, ctx, monkeypatch):
     """Where the qkv projection takes the 192- / 256-row kernels (more 128 x 128 tiles than compute units: from 641 rows on at
     this width) its epilogue rotates q and k and writes the cache rows itself; MOON_GEMM_NO_ROPE runs the projection and the
