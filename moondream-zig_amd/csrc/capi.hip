@@ -2,6 +2,7 @@
 // and their device-pointer twins.  Host-pointer ops stage operands into growable device buffers
 // (or use a registered resident weight), launch, copy the result back and wait.
 #include "moon_internal.hpp"
+#include <cstring>
 
 int launch_decode_attention_plain(moon_ctx *ctx, const half_t *q, const half_t *k, const half_t *v, half_t *out, size_t H,
                                   size_t kv_len, size_t D);
@@ -13,6 +14,16 @@ enum { ST_A = 0, ST_B = 1, ST_C = 2, ST_AUX = 3, ST_MASK = 4, ST_AUX2 = 5 };
 int stage_in(moon_ctx *ctx, int slot, const void *host, size_t bytes, void **dptr) {
     MOON_TRY(moon_grow(ctx, ctx->stage[slot], bytes ? bytes : 16));
     *dptr = ctx->stage[slot].ptr;
+    if (bytes && bytes <= MOON_PIN_BYTES) { // small operands through page-locked memory: the copy is queued, not waited for
+        if (!ctx->pin_up[slot] && hipHostMalloc(&ctx->pin_up[slot], MOON_PIN_BYTES, hipHostMallocDefault) != hipSuccess) {
+            ctx->pin_up[slot] = nullptr;
+            (void)hipGetLastError();
+        }
+        if (ctx->pin_up[slot]) {
+            memcpy(ctx->pin_up[slot], host, bytes);
+            host = ctx->pin_up[slot];
+        }
+    }
     if (bytes) MOON_HIP(ctx, hipMemcpyAsync(*dptr, host, bytes, hipMemcpyHostToDevice, ctx->stream));
     return MOON_OK;
 }
@@ -24,8 +35,17 @@ int stage_out(moon_ctx *ctx, int slot, size_t bytes, void **dptr) {
 }
 
 int fetch(moon_ctx *ctx, void *host, const void *dptr, size_t bytes) {
-    if (bytes) MOON_HIP(ctx, hipMemcpyAsync(host, dptr, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    void *dst = host;
+    if (bytes && bytes <= MOON_PIN_BYTES) {
+        if (!ctx->pin_down && hipHostMalloc(&ctx->pin_down, MOON_PIN_BYTES, hipHostMallocDefault) != hipSuccess) {
+            ctx->pin_down = nullptr;
+            (void)hipGetLastError();
+        }
+        if (ctx->pin_down) dst = ctx->pin_down;
+    }
+    if (bytes) MOON_HIP(ctx, hipMemcpyAsync(dst, dptr, bytes, hipMemcpyDeviceToHost, ctx->stream));
     MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (dst != host) memcpy(host, dst, bytes);
     return MOON_OK;
 }
 

@@ -82,6 +82,12 @@ extern "C" void moon_cleanup(moon_ctx *ctx) {
         if (b.ptr) (void)hipFree(b.ptr);
         b = GrowBuf();
     }
+    for (void *&p : ctx->pin_up) {
+        if (p) (void)hipHostFree(p);
+        p = nullptr;
+    }
+    if (ctx->pin_down) (void)hipHostFree(ctx->pin_down);
+    ctx->pin_down = nullptr;
     for (auto &b : ctx->work) {
         if (b.ptr) (void)hipFree(b.ptr);
         b = GrowBuf();

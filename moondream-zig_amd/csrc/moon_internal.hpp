@@ -20,6 +20,7 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
 // A device buffer that only ever grows; used for staging host-pointer calls and for workspaces.
+constexpr size_t MOON_PIN_BYTES = size_t(256) << 10;
 struct GrowBuf {
     void *ptr = nullptr;
     size_t cap = 0;
@@ -36,6 +37,11 @@ struct moon_ctx {
     char gemm_kernel[8] = ""; // moon_set_gemm_kernel / MOON_GEMM_KERNEL: a product kernel to take where the shape allows it ("": by shape)
     // staging for host-pointer ops: a, b, c, bias/aux, mask
     GrowBuf stage[6];
+    // page-locked host memory that the host-pointer entry points copy small operands and results through (allocated at first
+    // use, MOON_PIN_BYTES each, one per staging slot and one for results): a copy between device memory and the caller's
+    // pageable memory blocks the call for tens of microseconds.  Free again at the synchronisation that ends every such call.
+    void *pin_up[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    void *pin_down = nullptr;
     // kernel workspaces (split-K partials, attention partials, transposed B)
     GrowBuf work[4]; // 0: split-K partials, 1: decode-attention partials, 2: transposed operands, 3: split-K partials kept for a later launch
     // stand-alone decode attention in one launch: per-head "splits finished" counters behind the partials in work[1]

@@ -67,6 +67,10 @@ struct moon_text_model {
            *fc1 = nullptr, *mlp = nullptr, *logits = nullptr, *ln_last = nullptr;
     uint32_t *ids_dev = nullptr;   // [max_seq] prompt ids / generated ids
     uint32_t *ids_pinned = nullptr; // [max_seq] page-locked host memory the prompt ids are copied from (a copy from pageable memory blocks the call)
+    uint32_t *host_words = nullptr; // [64] page-locked: where the calls' small results land (error words, a token, the loop's state)
+    // page-locked staging for what the per-token calls move (a row of embeddings up; a hidden row, the logits, the ids down):
+    // a copy between device memory and the caller's pageable memory blocks the call for tens of microseconds
+    unsigned char *stage_up = nullptr, *stage_down = nullptr; // STAGE_BYTES each
     float *u_dev = nullptr;        // [max_seq] the sampling loop's random numbers, one per step
     uint32_t *state_dev = nullptr; // [0] position (KV length), [1] tokens recorded, [2] current token, [3] stopped, [4] eos id + 1 (record_token)
     size_t cur_len = 0, last_n = 0;
@@ -93,6 +97,8 @@ struct moon_text_model {
 
 namespace {
 
+constexpr size_t STAGE_BYTES = size_t(256) << 10; // (the logits of a 51,200-word vocabulary are 100 KB)
+
 __global__ void bump_pos_kernel(uint32_t *state) {
     if (!state[3]) state[0] += 1;
 }
@@ -115,6 +121,25 @@ int dalloc(moon_text_model *m, size_t bytes, void **p) {
     return MOON_OK;
 }
 template <class T> int dalloc_t(moon_text_model *m, size_t n, T **p) { return dalloc(m, n * sizeof(T), (void **)p); }
+
+// Host -> device, queued on the context's stream: small pieces go through the page-locked staging buffer (free again at the
+// call's final synchronisation; one use per call), large ones straight from the caller's memory.
+int copy_up(moon_text_model *m, void *dst_dev, const void *src_host, size_t bytes) {
+    if (bytes <= STAGE_BYTES && m->stage_up) {
+        memcpy(m->stage_up, src_host, bytes);
+        src_host = m->stage_up;
+    }
+    MOON_HIP(m->ctx, hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, m->ctx->stream));
+    return MOON_OK;
+}
+// Device -> host and the synchronisation that ends the call
+int copy_down_sync(moon_text_model *m, void *dst_host, const void *src_dev, size_t bytes) {
+    const bool staged = bytes <= STAGE_BYTES && m->stage_down;
+    MOON_HIP(m->ctx, hipMemcpyAsync(staged ? (void *)m->stage_down : dst_host, src_dev, bytes, hipMemcpyDeviceToHost, m->ctx->stream));
+    MOON_HIP(m->ctx, hipStreamSynchronize(m->ctx->stream));
+    if (staged) memcpy(dst_host, m->stage_down, bytes);
+    return MOON_OK;
+}
 
 struct Sizes {
     size_t L, d, ffn, V, H, D, S;
@@ -165,6 +190,9 @@ int alloc_all(moon_text_model *m) {
     MOON_TRY(dalloc_t(m, z.d, &m->ln_last));
     MOON_TRY(dalloc_t(m, z.S, &m->ids_dev));
     MOON_HIP(m->ctx, hipHostMalloc((void **)&m->ids_pinned, z.S * sizeof(uint32_t), hipHostMallocDefault));
+    MOON_HIP(m->ctx, hipHostMalloc((void **)&m->host_words, 64 * sizeof(uint32_t), hipHostMallocDefault));
+    MOON_HIP(m->ctx, hipHostMalloc((void **)&m->stage_up, STAGE_BYTES, hipHostMallocDefault));
+    MOON_HIP(m->ctx, hipHostMalloc((void **)&m->stage_down, STAGE_BYTES, hipHostMallocDefault));
     MOON_TRY(dalloc_t(m, z.S, &m->u_dev));
     MOON_TRY(dalloc_t(m, 8, &m->state_dev));
     MOON_TRY(launch_fill_uniform_u32(m->ctx, m->state_dev, 8, 0, 0, 1)); // zeros
@@ -202,7 +230,12 @@ void free_all(moon_text_model *m) {
     for (void *p : m->allocs) (void)hipFree(p);
     m->allocs.clear();
     if (m->ids_pinned) (void)hipHostFree(m->ids_pinned);
+    if (m->host_words) (void)hipHostFree(m->host_words);
+    if (m->stage_up) (void)hipHostFree(m->stage_up);
+    if (m->stage_down) (void)hipHostFree(m->stage_down);
+    m->stage_up = m->stage_down = nullptr;
     m->ids_pinned = nullptr;
+    m->host_words = nullptr;
 }
 
 // Counters, exchange buffers and error words of the fused decode kernels back to their initial state (fill kernels in
@@ -507,11 +540,12 @@ static int forward_rows_locked(moon_text_model *m, size_t n_ids) {
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->state_dev, (uint32_t)m->cur_len, 0u);
     MOON_HIP(ctx, hipGetLastError());
     // a single token takes the fused decode kernels, whose waits between workgroups are bounded: look at their error words
-    uint32_t wait_error[2] = {0, 0};
+    volatile uint32_t *wait_error = m->host_words; // (page-locked: the copies are queued like the kernels, one synchronisation for all)
+    wait_error[0] = wait_error[1] = 0;
     if (n_ids == 1 && m->fused) {
-        MOON_HIP(ctx, hipMemcpyAsync(&wait_error[0], m->layer_sync + m->cfg.n_layers * m->layer_sync_words, sizeof(uint32_t), hipMemcpyDeviceToHost,
+        MOON_HIP(ctx, hipMemcpyAsync(m->host_words, m->layer_sync + m->cfg.n_layers * m->layer_sync_words, sizeof(uint32_t), hipMemcpyDeviceToHost,
                                      ctx->stream));
-        MOON_HIP(ctx, hipMemcpyAsync(&wait_error[1], m->front_sync + m->cfg.n_layers * m->cfg.n_heads * 32, sizeof(uint32_t), hipMemcpyDeviceToHost,
+        MOON_HIP(ctx, hipMemcpyAsync(m->host_words + 1, m->front_sync + m->cfg.n_layers * m->cfg.n_heads * 32, sizeof(uint32_t), hipMemcpyDeviceToHost,
                                      ctx->stream));
     }
     MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -553,7 +587,7 @@ extern "C" int moon_text_forward_embeds(moon_text_model *m, const moon_f16 *embe
     if (m->cur_len + n_rows > m->cfg.max_seq)
         return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "text_forward_embeds: %zu + %zu rows > max_seq %zu (SequenceTooLong)", m->cur_len, n_rows, m->cfg.max_seq);
     MOON_HIP(ctx, hipSetDevice(ctx->device));
-    MOON_HIP(ctx, hipMemcpyAsync(m->hidden, embeds, n_rows * m->cfg.dim * sizeof(moon_f16), hipMemcpyHostToDevice, ctx->stream));
+    MOON_TRY(copy_up(m, m->hidden, embeds, n_rows * m->cfg.dim * sizeof(moon_f16)));
     return forward_rows_locked(m, n_rows);
 }
 
@@ -570,11 +604,9 @@ extern "C" int moon_text_embed(moon_text_model *m, const uint32_t *ids, size_t n
     // through buffers the session's state does not live in: the ids behind the loop's random numbers, the rows in the
     // MLP scratch (both are rewritten by whatever call uses them next)
     uint32_t *ids_tmp = reinterpret_cast<uint32_t *>(m->u_dev);
-    MOON_HIP(ctx, hipMemcpyAsync(ids_tmp, ids, n_ids * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
+    MOON_TRY(copy_up(m, ids_tmp, ids, n_ids * sizeof(uint32_t)));
     MOON_TRY(launch_embed(ctx, m->wte, ids_tmp, m->mlp, n_ids, m->cfg.dim));
-    MOON_HIP(ctx, hipMemcpyAsync(embeds, m->mlp, n_ids * m->cfg.dim * sizeof(moon_f16), hipMemcpyDeviceToHost, ctx->stream));
-    MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    return MOON_OK;
+    return copy_down_sync(m, embeds, m->mlp, n_ids * m->cfg.dim * sizeof(moon_f16));
 }
 
 extern "C" int moon_text_logits(moon_text_model *m, moon_f16 *logits) {
@@ -585,9 +617,7 @@ extern "C" int moon_text_logits(moon_text_model *m, moon_f16 *logits) {
     if (!m->last_n) return moon_fail(ctx, MOON_EINVAL, "text_logits: no forward pass yet");
     MOON_HIP(ctx, hipSetDevice(ctx->device));
     MOON_TRY(lm_head(m, m->last_n - 1));
-    MOON_HIP(ctx, hipMemcpyAsync(logits, m->logits, m->cfg.vocab * sizeof(moon_f16), hipMemcpyDeviceToHost, ctx->stream));
-    MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    return MOON_OK;
+    return copy_down_sync(m, logits, m->logits, m->cfg.vocab * sizeof(moon_f16));
 }
 
 extern "C" int moon_text_hidden(moon_text_model *m, moon_f16 *hidden, size_t n_rows) {
@@ -596,9 +626,7 @@ extern "C" int moon_text_hidden(moon_text_model *m, moon_f16 *hidden, size_t n_r
     std::lock_guard<std::mutex> lock(ctx->mu);
     if (!hidden) return moon_fail(ctx, MOON_EINVAL, "text_hidden: null output");
     if (n_rows > m->last_n) return moon_fail(ctx, MOON_EINVAL_DIM, "text_hidden: %zu rows requested, last forward had %zu", n_rows, m->last_n);
-    MOON_HIP(ctx, hipMemcpyAsync(hidden, m->hidden, n_rows * m->cfg.dim * sizeof(moon_f16), hipMemcpyDeviceToHost, ctx->stream));
-    MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    return MOON_OK;
+    return copy_down_sync(m, hidden, m->hidden, n_rows * m->cfg.dim * sizeof(moon_f16));
 }
 
 // MOON_DECODE_TRACE: where the workgroups of the last whole-layer launch spent their time, by role (microseconds after
@@ -647,7 +675,7 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
     if (m->cur_len + n_steps > m->cfg.max_seq)
         return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "text_greedy: %zu + %zu tokens > max_seq %zu (SequenceTooLong)", m->cur_len, n_steps, m->cfg.max_seq);
     MOON_HIP(ctx, hipSetDevice(ctx->device));
-    if (sampling) MOON_HIP(ctx, hipMemcpyAsync(m->u_dev, u, n_steps * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    if (sampling) MOON_TRY(copy_up(m, m->u_dev, u, n_steps * sizeof(float)));
     uint32_t *state = m->state_dev;
     hipLaunchKernelGGL(start_loop_kernel, dim3(1), dim3(1), 0, ctx->stream, state, (uint32_t)m->cur_len, eos_plus1);
     MOON_HIP(ctx, hipGetLastError());
@@ -724,22 +752,28 @@ static int greedy_locked(moon_text_model *m, size_t n_steps, uint32_t *out_ids, 
             p.kinds.clear();
         }
         if (eos_plus1 && (step + 1) % EOS_CHUNK == 0 && step + 1 < n_steps) { // has the end-of-sequence token come up?
-            uint32_t st[4];
-            MOON_HIP(ctx, hipMemcpyAsync(st, state, sizeof(st), hipMemcpyDeviceToHost, ctx->stream));
+            volatile uint32_t *st = m->host_words + 16;
+            MOON_HIP(ctx, hipMemcpyAsync(m->host_words + 16, state, 4 * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
             MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
             if (st[3]) break;
         }
     }
-    uint32_t front_error = 0;
-    uint32_t final_state[4] = {0, (uint32_t)n_steps, 0, 0};
-    if (eos_plus1) MOON_HIP(ctx, hipMemcpyAsync(final_state, state, sizeof(final_state), hipMemcpyDeviceToHost, ctx->stream));
-    MOON_HIP(ctx, hipMemcpyAsync(out_ids, m->ids_dev, n_steps * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    // everything the call brings back lands in page-locked memory (queued like the kernels), one synchronisation for all of it
+    volatile uint32_t *words = m->host_words;
+    words[20] = 0; words[21] = (uint32_t)n_steps; words[22] = 0; words[23] = 0; // the loop's final state where no copy is asked for
+    words[24] = 0;                                                            // the error word
+    if (eos_plus1) MOON_HIP(ctx, hipMemcpyAsync(m->host_words + 20, state, 4 * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    const bool ids_staged = n_steps * sizeof(uint32_t) <= STAGE_BYTES;
+    MOON_HIP(ctx, hipMemcpyAsync(ids_staged ? (void *)m->stage_down : (void *)out_ids, m->ids_dev, n_steps * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
     if (use_layer)
-        MOON_HIP(ctx, hipMemcpyAsync(&front_error, m->layer_sync + m->cfg.n_layers * m->layer_sync_words, sizeof(front_error), hipMemcpyDeviceToHost,
+        MOON_HIP(ctx, hipMemcpyAsync(m->host_words + 24, m->layer_sync + m->cfg.n_layers * m->layer_sync_words, sizeof(uint32_t), hipMemcpyDeviceToHost,
                                      ctx->stream));
     if (use_front)
-        MOON_HIP(ctx, hipMemcpyAsync(&front_error, m->front_sync + m->cfg.n_layers * m->cfg.n_heads * 32, sizeof(front_error), hipMemcpyDeviceToHost, ctx->stream));
+        MOON_HIP(ctx, hipMemcpyAsync(m->host_words + 24, m->front_sync + m->cfg.n_layers * m->cfg.n_heads * 32, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
     MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (ids_staged) memcpy(out_ids, m->stage_down, n_steps * sizeof(uint32_t));
+    const uint32_t front_error = words[24];
+    const uint32_t final_state[4] = {words[20], words[21], words[22], words[23]};
     if (front_error != 0) {
         // Workgroups that gave up skipped their counter updates and the cache append of their position: the counters
         // are cleared here, the cache and the position stay unusable until moon_text_reset.
@@ -816,8 +850,9 @@ extern "C" int moon_text_next_token(moon_text_model *m, const moon_sampling_conf
     uint32_t *out = m->state_dev + 5; // a word of the loop's state that the loop itself does not use
     if (!cfg || cfg->method == MOON_SAMPLE_GREEDY) MOON_TRY(launch_argmax(ctx, m->logits, m->cfg.vocab, out));
     else MOON_TRY(launch_sample(ctx, m->logits, m->cfg.vocab, cfg, u, nullptr, nullptr, nullptr, out));
-    MOON_HIP(ctx, hipMemcpyAsync(token, out, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    MOON_HIP(ctx, hipMemcpyAsync(m->host_words + 8, out, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
     MOON_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    *token = const_cast<volatile uint32_t *>(m->host_words)[8];
     return MOON_OK;
 }
 
