@@ -653,40 +653,19 @@ __device__ __forceinline__ bool wait_reached(uint32_t *word, uint32_t target, ui
 }
 
 
-// 16 bytes, device-coherent, waited for on the spot (p 16-byte aligned)
-__device__ __forceinline__ u32x4 ld_u128_coh(const void *p) {
-    u32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    return v;
-}
-// dot of the loaded row (group slot 0) with a vector that lives in LDS, pieces in the same order as RowGroups::consume
-template <int CH>
-__device__ __forceinline__ float dot_row_lds(const u32x4 (&w)[CH], const half_t *x_lds, int K, int lane) {
-    float s = 0.0f;
-#pragma unroll
-    for (int c = 0; c < CH; c++) {
-        const int g = c * 64 + lane;
-        u32x4 xv = u32x4{0, 0, 0, 0};
-        if (g < (K >> 3)) xv = *reinterpret_cast<const u32x4 *>(x_lds + size_t(g) * 8);
-        s = dot8(w[c], xv, s);
-    }
-    return wave_sum(s);
-}
-
 // FC1_GROUP: fc1 rows a wavefront requests together.  The fewer bytes a compute unit has queued, the sooner the small
 // dependent accesses of the attention chain issued from it are served (two measured 3 % slower than one).
 // PF: 32-key steps of an attention task whose K and V rows are requested before the wait for q (decode_attn_prefetch); the
 // host picks the instantiation that covers a split at the launch's position.
 template <int CH_D, int CH_F, int FC1_GROUP, int PF>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void decode_layer_kernel(LayerArgs a) {
-    extern __shared__ __attribute__((aligned(16))) half_t smem[]; // [d] LayerNorm output, later attn; then [ffn] fc1
+    extern __shared__ __attribute__((aligned(16))) half_t smem[]; // [d] LayerNorm output; then [ffn] fc1
     __shared__ float s_red[16];
     __shared__ int s_flag;
-    constexpr int RG = 4;
     const LnGemvArgs &p = a.g;
     half_t *s_ln = smem, *s_fc1 = smem + p.d;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n_waves = gridDim.x * 4, gw = blockIdx.x * 4 + wave;
+    const int gw = blockIdx.x * 4 + wave;
     const int n_attn = a.H * DEC_SPLITS, n_out = (p.d + 3) / 4;
     const int b = blockIdx.x;
     const bool attn_wg = b < n_attn, out_wg = !attn_wg && b < n_attn + n_out;
@@ -827,30 +806,45 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const unsigned fc1_leaves = n_fc1_wgs < LAYER_FC1_LEAVES ? n_fc1_wgs : LAYER_FC1_LEAVES;
     if (!wait_reached(a.sync + LAYER_SYNC_FC1_ROOT * LAYER_LINE, a.generation * fc1_leaves, a.error, &s_flag)) return;
     stamp(3); // all fc1 rows written
-    for (int i = tid; i < a.ffn / 4; i += 256) // fc1 vector, 8 bytes per coherent load
-        reinterpret_cast<unsigned long long *>(s_fc1)[i] = ld_u64_coh(p.y2 + size_t(i) * 4);
+    // fc1 vector, 8 bytes per coherent load: the waits space out the requests (0.628 ms per token with 16-byte loads, 0.598 as it
+    // is; an agent-scope acquire followed by plain loads, so that the die's L2 serves 63 of its 64 workgroups: 0.91 ms)
+    for (int i = tid; i < a.ffn / 4; i += 256) reinterpret_cast<unsigned long long *>(s_fc1)[i] = ld_u64_coh(p.y2 + size_t(i) * 4);
+    lds_barrier();
+    // the fc2 row's product is taken before the wait for the heads (the fc1 vector is complete microseconds before the last head):
+    // what follows that wait is the launch's last hop
+    float dot_f = 0.0f; // pieces in the same order as RowGroups::consume
+    if (have_row) {
+#pragma unroll
+        for (int c = 0; c < CH_F; c++) {
+            const int g = c * 64 + lane;
+            // (ffn is a multiple of 512 here, decode_layer_supported: every lane has its piece.  A guarded read would put each
+            // piece behind a branch of its own, and the compiler then keeps all sixteen in registers that are not there.)
+            const u32x4 xg = *reinterpret_cast<const u32x4 *>(s_fc1 + size_t(g) * 8);
+            dot_f = dot8(fc2_row.w[0][c], xg, dot_f);
+        }
+        dot_f = wave_sum(dot_f);
+    }
     if (!wait_reached(a.sync + LAYER_SYNC_HEADS_DONE * LAYER_LINE, a.generation * (uint32_t)a.H, a.error, &s_flag)) return;
     stamp(4); // all heads merged
-    half_t *s_attn = s_ln; // the LayerNorm output is no longer needed
-    // (one 16-byte load per thread: this copy is the last hop of the launch.  The fc1 vector above is better off in 8-byte
-    // loads, whose waits space out the requests: 0.628 ms per token with 16-byte ones there, 0.598 as it is, 0.602 with both in
-    // 8-byte loads; an agent-scope acquire followed by plain loads, so that the die's L2 serves 63 of its 64 workgroups: 0.91 ms)
-    for (int i = tid; i < p.d / 8; i += 256) reinterpret_cast<u32x4 *>(s_attn)[i] = ld_u128_coh(a.attn_out + size_t(i) * 8);
-    lds_barrier();
     if (!have_row) return;
     const half_t bias_o = __builtin_bit_cast(half_t, (unsigned short)bias_o_bits), bias_f = __builtin_bit_cast(half_t, (unsigned short)bias_f_bits);
     const half_t hid = __builtin_bit_cast(half_t, (unsigned short)hid_bits);
-    const float dot_o = dot_row_lds<CH_D>(out_row.w[0], s_attn, p.d, lane);
-    float dot_f = 0.0f; // dot_row_lds without its guards
+    // The attention output goes straight into each wavefront's registers, a lane fetching the pieces that meet its pieces of the
+    // out_proj row (d is a multiple of 512: every lane has them): four times the requests of one copy into LDS per workgroup, but
+    // no LDS round trip and no barrier behind the last wait (0.5831 against 0.5869 ms per token).  Same pieces in the same order
+    // as RowGroups::consume.
+    float dot_o = 0.0f;
+    {
+        u32x4 xa[CH_D];
 #pragma unroll
-    for (int c = 0; c < CH_F; c++) {
-        const int g = c * 64 + lane;
-        // (ffn is a multiple of 512 here, decode_layer_supported: every lane has its piece.  A guarded read would put each
-        // piece behind a branch of its own, and the compiler then keeps all sixteen in registers that are not there.)
-        const u32x4 xg = *reinterpret_cast<const u32x4 *>(s_fc1 + size_t(g) * 8);
-        dot_f = dot8(fc2_row.w[0][c], xg, dot_f);
+        for (int c = 0; c < CH_D; c++)
+            asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(xa[c]) : "v"(a.attn_out + size_t(c * 64 + lane) * 8) : "memory");
+#pragma unroll
+        for (int c = 0; c < CH_D; c++) asm volatile("s_waitcnt vmcnt(0)" : "+v"(xa[c])::"memory");
+#pragma unroll
+        for (int c = 0; c < CH_D; c++) dot_o = dot8(out_row.w[0][c], xa[c], dot_o);
+        dot_o = wave_sum(dot_o);
     }
-    dot_f = wave_sum(dot_f);
     if (lane == 0) {
         const half_t ao = apply_epilogue_v<MOON_EPI_BIAS>(dot_o, bias_o);
         const half_t m = apply_epilogue_v<MOON_EPI_BIAS>(dot_f, bias_f);
