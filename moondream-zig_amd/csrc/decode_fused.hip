@@ -806,9 +806,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const unsigned fc1_leaves = n_fc1_wgs < LAYER_FC1_LEAVES ? n_fc1_wgs : LAYER_FC1_LEAVES;
     if (!wait_reached(a.sync + LAYER_SYNC_FC1_ROOT * LAYER_LINE, a.generation * fc1_leaves, a.error, &s_flag)) return;
     stamp(3); // all fc1 rows written
-    // fc1 vector, 8 bytes per coherent load: the waits space out the requests (0.628 ms per token with 16-byte loads, 0.598 as it
-    // is; an agent-scope acquire followed by plain loads, so that the die's L2 serves 63 of its 64 workgroups: 0.91 ms)
-    for (int i = tid; i < a.ffn / 4; i += 256) reinterpret_cast<unsigned long long *>(s_fc1)[i] = ld_u64_coh(p.y2 + size_t(i) * 4);
+    // The fc1 vector, one 16-byte load per thread at a time, each waited for (requested two or four at a time the copies of the 512
+    // workgroups pile up on the same 128 lines: 0.593 / 0.610 against 0.578 ms per token).  The loads are workgroup-scope ones
+    // (sc0), which the die's L2 serves: every byte of the vector was written through to memory (sc1 stores) before the counter
+    // this workgroup has just waited for was raised, and no workgroup reads a line of it before that, so the first of a die's 64
+    // output workgroups to ask takes the line from memory as it is and the others share it.  Device-scope loads, which pass
+    // the L2, cost 8 MB of fabric traffic per launch at the moment the weight stream ends (0.585 ms; in 8-byte pieces).
+    for (int i = tid; i < a.ffn / 8; i += 256) {
+        u32x4 v;
+        asm volatile("global_load_dwordx4 %0, %1, off sc0\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p.y2 + size_t(i) * 8) : "memory");
+        reinterpret_cast<u32x4 *>(s_fc1)[i] = v;
+    }
     lds_barrier();
     // the fc2 row's product is taken before the wait for the heads (the fc1 vector is complete microseconds before the last head):
     // what follows that wait is the launch's last hop
@@ -832,13 +840,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     // The attention output goes straight into each wavefront's registers, a lane fetching the pieces that meet its pieces of the
     // out_proj row (d is a multiple of 512: every lane has them): four times the requests of one copy into LDS per workgroup, but
     // no LDS round trip and no barrier behind the last wait (0.5831 against 0.5869 ms per token).  Same pieces in the same order
-    // as RowGroups::consume.
+    // as RowGroups::consume.  Workgroup-scope loads through the die's L2, like the fc1 vector's: the heads were written through
+    // before the counter rose.
     float dot_o = 0.0f;
     {
         u32x4 xa[CH_D];
 #pragma unroll
         for (int c = 0; c < CH_D; c++)
-            asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(xa[c]) : "v"(a.attn_out + size_t(c * 64 + lane) * 8) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off sc0" : "=v"(xa[c]) : "v"(a.attn_out + size_t(c * 64 + lane) * 8) : "memory");
 #pragma unroll
         for (int c = 0; c < CH_D; c++) asm volatile("s_waitcnt vmcnt(0)" : "+v"(xa[c])::"memory");
 #pragma unroll

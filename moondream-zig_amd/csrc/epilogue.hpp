@@ -90,10 +90,6 @@ template <bool COH> __device__ __forceinline__ void st_f(float *p, float v) {
 }
 __device__ __forceinline__ int ld_i_coh(const int *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_i_coh(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-// 8 bytes (4 halfs) at once; p must be 8-byte aligned
-__device__ __forceinline__ unsigned long long ld_u64_coh(const void *p) {
-    return __hip_atomic_load(reinterpret_cast<const unsigned long long *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 // 64-lane reductions on the DPP cross-lane path (no LDS crossbar): quad swaps (xor 1, xor 2), mirror within
 // 8 lanes, mirror within the 16-lane row, then the four row results are read out and combined.  Fixed order,
