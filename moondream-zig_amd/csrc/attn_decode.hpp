@@ -98,7 +98,8 @@ __device__ __forceinline__ void decode_attn_task(const half_t *__restrict__ qkv,
                                                  half_t *__restrict__ cv, const float *__restrict__ table,
                                                  float *__restrict__ partial, int H, int rot_dim, int max_seq, int pos_real,
                                                  int h, int split, const DecodeAttnPrefetch<PF> &pf, uint32_t *head_count = nullptr,
-                                                 uint32_t count_target = 0, half_t *merged_out = nullptr, uint32_t *done_count = nullptr) {
+                                                 uint32_t count_target = 0, half_t *merged_out = nullptr, uint32_t *done_count = nullptr,
+                                                 int done_copies = 1, int done_stride = 0) {
     static_assert(D == 64, "one 16-byte granule per lane, 8 lanes per key");
     __shared__ float sq[D];
     __shared__ __attribute__((aligned(16))) half_t sk_new[D];
@@ -247,7 +248,8 @@ __device__ __forceinline__ void decode_attn_task(const half_t *__restrict__ qkv,
         if (s_last && wave == 0) { // t < D: the merged head, then (once acknowledged) the head is counted as done
             st_h<true>(merged_out + h * D + t, decode_attn_merge<D, true>(partial + size_t(h) * DEC_SPLITS * (D + 2), t));
             __builtin_amdgcn_s_waitcnt(0);
-            if (t == 0 && done_count) __hip_atomic_fetch_add(done_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // (done_copies copies of the counter, done_stride words apart: a lane each)
+            if (t < done_copies && done_count) __hip_atomic_fetch_add(done_count + t * done_stride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }

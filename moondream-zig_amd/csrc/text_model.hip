@@ -883,7 +883,7 @@ extern "C" int moon_text_debug_raise_wait_error(moon_text_model *m) {
     std::lock_guard<std::mutex> lock(ctx->mu);
     const Sizes z = sizes(m->cfg);
     MOON_HIP(ctx, hipSetDevice(ctx->device));
-    // the word before each error word is the unused tail of a counter line: writes {0, 1} to (tail, error word)
+    // the word before each error word is unused (the tail of a counter line, or of the last counter copy): writes {0, 1} to (tail, error word)
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->layer_sync + z.L * m->layer_sync_words - 1, 0u, 1u);
     MOON_HIP(ctx, hipGetLastError());
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx->stream, m->front_sync + z.L * z.H * 32 - 1, 0u, 1u);
