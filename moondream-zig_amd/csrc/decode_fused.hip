@@ -820,16 +820,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const unsigned fc1_leaves = n_fc1_wgs < LAYER_FC1_LEAVES ? n_fc1_wgs : LAYER_FC1_LEAVES;
     if (!wait_reached(bcast + (LAYER_BCAST_FC1 * LAYER_COPIES + b % LAYER_COPIES) * LAYER_COPY_STRIDE, a.generation * fc1_leaves, a.error, &s_flag)) return;
     stamp(3); // all fc1 rows written
-    // The fc1 vector, one 16-byte load per thread at a time, each waited for (requested two or four at a time the copies of the 512
-    // workgroups pile up on the same 128 lines: 0.593 / 0.610 against 0.578 ms per token).  The loads are workgroup-scope ones
-    // (sc0), which the die's L2 serves: every byte of the vector was written through to memory (sc1 stores) before the counter
-    // this workgroup has just waited for was raised, and no workgroup reads a line of it before that, so the first of a die's 64
-    // output workgroups to ask takes the line from memory as it is and the others share it.  Device-scope loads, which pass
-    // the L2, cost 8 MB of fabric traffic per launch at the moment the weight stream ends (0.585 ms; in 8-byte pieces).
-    for (int i = tid; i < a.ffn / 8; i += 256) {
-        u32x4 v;
-        asm volatile("global_load_dwordx4 %0, %1, off sc0\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p.y2 + size_t(i) * 8) : "memory");
-        reinterpret_cast<u32x4 *>(s_fc1)[i] = v;
+    // The fc1 vector: four 16-byte loads per thread, one round trip.  They are workgroup-scope loads (sc0), which the die's L2
+    // serves: every byte of the vector was written through to memory (sc1 stores) before the counter this workgroup has just
+    // waited for was raised, and no workgroup reads a line of it before that, so the first of a die's 64 output workgroups to
+    // ask takes the line from memory as it is and the others share it.  Device-scope loads, which pass the L2, cost 8 MB of
+    // fabric traffic per launch at the moment the weight stream ends (0.585 against 0.578 ms per token, in 8-byte pieces, each
+    // waited for).  (While all 512 output workgroups polled one counter line, anything that brought them to the next wait
+    // sooner made the launch longer, this copy in one round trip included: 0.610 ms.)
+    {
+        static_assert(CH_F % 4 == 0, "ffn = 512 CH_F halfs in 16-byte pieces over 256 threads");
+        u32x4 v[CH_F / 4];
+#pragma unroll
+        for (int k = 0; k < CH_F / 4; k++)
+            asm volatile("global_load_dwordx4 %0, %1, off sc0" : "=v"(v[k]) : "v"(p.y2 + size_t(tid + 256 * k) * 8) : "memory");
+#pragma unroll
+        for (int k = 0; k < CH_F / 4; k++) asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[k])::"memory");
+#pragma unroll
+        for (int k = 0; k < CH_F / 4; k++) reinterpret_cast<u32x4 *>(s_fc1)[tid + 256 * k] = v[k];
     }
     lds_barrier();
     // the fc2 row's product is taken before the wait for the heads (the fc1 vector is complete microseconds before the last head):
