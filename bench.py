@@ -36,11 +36,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense FP16
 
-# HBM bytes per launch of the dominant kernel (decode_layer_kernel) from rocprofv3 counters: FETCH_SIZE 52814.71 KiB x
-# 1.99984 plus WRITE_SIZE 628.00 KiB x 1.0, the factors being what the same counters read for the 256 MiB copies of
+# HBM bytes per launch of the dominant kernel (decode_layer_kernel) from rocprofv3 counters: FETCH_SIZE 52846.23 KiB x
+# 1.99984 plus WRITE_SIZE 754.00 KiB x 1.0, the factors being what the same counters read for the 256 MiB copies of
 # --calibrate-copy (profiles/decode_kernels_hbm_traffic_pmc.txt).  A measured constant, not a live reading; it belongs
 # to the default decode mode.
-TRAFFIC_BYTES_PER_LAUNCH = 108_798_717
+TRAFFIC_BYTES_PER_LAUNCH = 108_992_459
 
 PREFILL = 768
 D, FFN, H, HD, L, V = 2048, 8192, 32, 64, 24, 51200
