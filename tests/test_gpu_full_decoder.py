@@ -41,3 +41,23 @@ def test_full_size_greedy_ids_match_oracle_for_64_steps(moon, O, ctx):
         assert dev.greedy(64).tolist() == want, f"decode mode {mode}"
     assert dev.position == 768 + 64
     dev.close()
+
+
+def test_the_cache_filled_token_by_token_in_the_default_mode_matches_the_wait_free_mode(moon, O, ctx):
+    """1,983 greedy tokens from a 64-token prompt, to the end of the 2048-entry cache: the default mode (one kernel per layer,
+    whose workgroups hand the qkv rows, the fc1 vector and the attention output to each other inside the launch, the
+    last two through the die's L2 and behind counters that exist in copies) against mode 2 (three kernels per layer,
+    no exchange inside a launch).  One stale or early read of an exchanged vector anywhere in 47,592 layer launches
+    would change the hidden state and with it the ids from there on."""
+    dev = moon.text_model.TextModel(moon.text_model.default_config(), seed=0, std=0.02, ctx=ctx)
+    ids = O.fill_uniform_u32(64, 0, 50, O.TEXT_CFG["vocab"])
+    out = {}
+    for mode in (0, 2):
+        dev.set_decode_mode(mode)
+        dev.reset()
+        dev.forward(ids)
+        out[mode] = dev.greedy(2047 - len(ids))
+    dev.close()
+    assert len(out[0]) == 1983
+    differ = np.flatnonzero(out[0] != out[2])
+    assert differ.size == 0, f"first difference at step {int(differ[0])} (position {64 + int(differ[0])})"
