@@ -152,8 +152,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
     int item = (int)(blockIdx.y * gridDim.x + blockIdx.x);
     const int n_items = (int)(gridDim.x * gridDim.y);
     if (n_items % 8 == 0) item = (item % 8) * (n_items / 8) + item / 8;
-    const int h = item / (int)gridDim.x, bx = item % (int)gridDim.x;
-    // late query blocks see the most keys: start them first
+    int h = item / (int)gridDim.x, bx = item % (int)gridDim.x;
+    // Late query blocks see the most keys: start them first.  Where a die's share is whole heads, its workgroups walk the
+    // query blocks of all its heads together (block 23 of heads 0-3, block 22 of heads 0-3, ...): what is still to start when
+    // the first workgroups leave is then the lightest blocks of every head, not all of the last head's.
+    if (causal && n_items % 8 == 0 && (n_items / 8) % (int)gridDim.x == 0) {
+        const int per_die = n_items / 8, heads_per_die = per_die / (int)gridDim.x, j = item % per_die;
+        h = (item / per_die) * heads_per_die + j % heads_per_die;
+        bx = j / heads_per_die;
+    }
     const int qb = causal ? (int)gridDim.x - 1 - bx : bx;
     const int q0 = qb * FA_Q;
     half_t *Ks = smem + wave * C::WAVE_HALFS;
