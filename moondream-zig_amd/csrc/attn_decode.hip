@@ -35,7 +35,7 @@ __global__ void decode_attn_merge_kernel(const float *__restrict__ partial, half
 
 int launch_decode_attention_merged(moon_ctx *ctx, const half_t *qkv, half_t *cache_k, half_t *cache_v, const float *table, float *partial,
                                    half_t *out, uint32_t *head_count, uint32_t count_target, size_t H, size_t D, size_t rot_dim,
-                                   size_t max_seq, size_t pos, const uint32_t *pos_dev);
+                                   size_t max_seq, size_t pos, const uint32_t *pos_dev, size_t head_stride = 1);
 
 int launch_decode_attention(moon_ctx *ctx, const half_t *qkv, half_t *cache_k, half_t *cache_v, const float *table, half_t *out,
                             size_t H, size_t D, size_t rot_dim, size_t max_seq, size_t pos, const uint32_t *pos_dev) {
@@ -46,17 +46,20 @@ int launch_decode_attention(moon_ctx *ctx, const half_t *qkv, half_t *cache_k, h
     // One launch: the split that finishes a head last merges it (the kernel of the text session's three-kernel decode
     // mode).  Its per-head counters sit behind the partials and count up from launch to launch.
     const size_t partial_bytes = (H * DEC_SPLITS * (D + 2) * sizeof(float) + 255) & ~size_t(255);
-    MOON_TRY(moon_grow(ctx, ctx->work[1], partial_bytes + H * sizeof(uint32_t)));
+    // (the heads' counters 4,352 bytes apart: all splits of all heads count in at about the same time, and atomics on one line
+    // are served one after the other)
+    constexpr size_t HEAD_STRIDE = 1088;
+    MOON_TRY(moon_grow(ctx, ctx->work[1], partial_bytes + H * HEAD_STRIDE * sizeof(uint32_t)));
     float *partial = (float *)ctx->work[1].ptr;
     uint32_t *head_count = reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(ctx->work[1].ptr) + partial_bytes);
     if (ctx->attn_cnt_buf != (void *)head_count || ctx->attn_cnt_heads != H || ctx->attn_cnt_launches >= (1u << 28)) {
-        MOON_TRY(launch_fill_uniform_u32(ctx, head_count, H, 0, 0, 1)); // zeros, in stream order
+        MOON_TRY(launch_fill_uniform_u32(ctx, head_count, H * HEAD_STRIDE, 0, 0, 1)); // zeros, in stream order
         ctx->attn_cnt_buf = head_count;
         ctx->attn_cnt_heads = H;
         ctx->attn_cnt_launches = 0;
     }
     const uint32_t target = ++ctx->attn_cnt_launches * (uint32_t)DEC_SPLITS;
-    return launch_decode_attention_merged(ctx, qkv, cache_k, cache_v, table, partial, out, head_count, target, H, D, rot_dim, max_seq, pos, pos_dev);
+    return launch_decode_attention_merged(ctx, qkv, cache_k, cache_v, table, partial, out, head_count, target, H, D, rot_dim, max_seq, pos, pos_dev, HEAD_STRIDE);
 }
 
 // q[H,64] already rotated, k,v[H][kv_len][64] contiguous: singleMaskedSDPA with an all-true mask.

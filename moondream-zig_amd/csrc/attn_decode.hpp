@@ -99,7 +99,7 @@ __device__ __forceinline__ void decode_attn_task(const half_t *__restrict__ qkv,
                                                  float *__restrict__ partial, int H, int rot_dim, int max_seq, int pos_real,
                                                  int h, int split, const DecodeAttnPrefetch<PF> &pf, uint32_t *head_count = nullptr,
                                                  uint32_t count_target = 0, half_t *merged_out = nullptr, uint32_t *done_count = nullptr,
-                                                 int done_copies = 1, int done_stride = 0) {
+                                                 int done_copies = 1, int done_stride = 0, int head_stride = 1) {
     static_assert(D == 64, "one 16-byte granule per lane, 8 lanes per key");
     __shared__ float sq[D];
     __shared__ __attribute__((aligned(16))) half_t sk_new[D];
@@ -240,7 +240,7 @@ __device__ __forceinline__ void decode_attn_task(const half_t *__restrict__ qkv,
         if (wave == 0) {
             __builtin_amdgcn_s_waitcnt(0); // vmcnt(0): the partial has reached memory
             if (t == 0) {
-                const uint32_t old = __hip_atomic_fetch_add(head_count + h, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const uint32_t old = __hip_atomic_fetch_add(head_count + size_t(h) * head_stride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 s_last = (old + 1 == count_target) ? 1 : 0;
             }
         }

@@ -959,13 +959,14 @@ __global__ __launch_bounds__(256) void decode_attn_merged_kernel(const half_t *_
                                                                   half_t *__restrict__ cv, const float *__restrict__ table,
                                                                   float *__restrict__ partial, half_t *__restrict__ out,
                                                                   uint32_t *head_count, uint32_t count_target, int H, int rot_dim,
-                                                                  int max_seq, int pos_arg, const uint32_t *__restrict__ pos_dev) {
+                                                                  int max_seq, int pos_arg, const uint32_t *__restrict__ pos_dev, int head_stride) {
     const int pos = pos_dev ? (int)*pos_dev : pos_arg;
     const int h = blockIdx.x / DEC_SPLITS, split = blockIdx.x % DEC_SPLITS;
     DecodeAttnPrefetch<PF> pf;
     decode_attn_prefetch<D, PF>(pf, ck, cv, max_seq, pos, true, h, split);
     // device-coherent partials and a per-head counter: whichever split finishes a head last merges it
-    decode_attn_task<D, true, true, PF>(qkv, ck, cv, table, partial, H, rot_dim, max_seq, pos, h, split, pf, head_count, count_target, out);
+    decode_attn_task<D, true, true, PF>(qkv, ck, cv, table, partial, H, rot_dim, max_seq, pos, h, split, pf, head_count, count_target, out, nullptr, 1, 0,
+                                        head_stride);
 }
 
 // sampling.argmax (sampling.zig:257-273) + bookkeeping of the greedy loop: state[2] = token, out_ids[state[1]++] = token.
@@ -1274,16 +1275,16 @@ int launch_decode_out_fc2(moon_ctx *ctx, const half_t *attn, const half_t *fc1, 
 // head_count: H persistent counters of this layer; count_target = DEC_SPLITS x (number of launches on them so far, this one included)
 int launch_decode_attention_merged(moon_ctx *ctx, const half_t *qkv, half_t *cache_k, half_t *cache_v, const float *table, float *partial,
                                    half_t *out, uint32_t *head_count, uint32_t count_target, size_t H, size_t D, size_t rot_dim,
-                                   size_t max_seq, size_t pos, const uint32_t *pos_dev) {
+                                   size_t max_seq, size_t pos, const uint32_t *pos_dev, size_t head_stride) {
     if (D != 64) return moon_fail(ctx, MOON_EINVAL_DIM, "decode attention: head_dim %zu unsupported (64 only)", D);
     if (max_seq > 2048 || pos >= max_seq) return moon_fail(ctx, MOON_ESEQ_TOO_LONG, "decode attention: pos %zu >= max_seq %zu (limit 2048)", pos, max_seq);
     // (two prefetch depths: up to 4 steps of 32 keys per split, which is 896 cached keys, and everything beyond; see launch_decode_layer)
     if ((pos + DEC_SPLITS - 2) / (DEC_SPLITS - 1) <= 128)
         hipLaunchKernelGGL((decode_attn_merged_kernel<64, 4>), dim3((unsigned)(H * DEC_SPLITS)), dim3(256), 0, ctx->stream, qkv, cache_k, cache_v, table,
-                           partial, out, head_count, count_target, (int)H, (int)rot_dim, (int)max_seq, (int)pos, pos_dev);
+                           partial, out, head_count, count_target, (int)H, (int)rot_dim, (int)max_seq, (int)pos, pos_dev, (int)head_stride);
     else
         hipLaunchKernelGGL((decode_attn_merged_kernel<64, 10>), dim3((unsigned)(H * DEC_SPLITS)), dim3(256), 0, ctx->stream, qkv, cache_k, cache_v, table,
-                           partial, out, head_count, count_target, (int)H, (int)rot_dim, (int)max_seq, (int)pos, pos_dev);
+                           partial, out, head_count, count_target, (int)H, (int)rot_dim, (int)max_seq, (int)pos, pos_dev, (int)head_stride);
     MOON_HIP(ctx, hipGetLastError());
     MOON_NOTE_KERNEL(ctx, "decode_attn_merged_kernel<64> %d workgroups", (int)(H * DEC_SPLITS));
     return MOON_OK;

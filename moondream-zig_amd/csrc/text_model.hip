@@ -20,7 +20,7 @@ int launch_decode_out_fc2(moon_ctx *ctx, const half_t *attn, const half_t *fc1, 
                           const half_t *b2, half_t *hidden, const half_t *hidden_src, const uint32_t *token, size_t d, size_t ffn);
 int launch_decode_attention_merged(moon_ctx *ctx, const half_t *qkv, half_t *cache_k, half_t *cache_v, const float *table, float *partial,
                                    half_t *out, uint32_t *head_count, uint32_t count_target, size_t H, size_t D, size_t rot_dim,
-                                   size_t max_seq, size_t pos, const uint32_t *pos_dev);
+                                   size_t max_seq, size_t pos, const uint32_t *pos_dev, size_t head_stride = 1);
 int launch_argmax_record(moon_ctx *ctx, const half_t *logits, size_t n, uint32_t *state, uint32_t *out_ids);
 size_t decode_lm_head_words(moon_ctx *ctx);
 int launch_decode_lm_head(moon_ctx *ctx, const half_t *x, const half_t *gamma, const half_t *beta, float eps, size_t d, const half_t *W,
